@@ -1,0 +1,261 @@
+"""Benchmark of the OLMoE MoE layer (64 experts, top-8, 2048 -> 1024 -> 2048, fp16) on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--tokens N] [--mode auto|gemv|gemm]
+    python bench.py --sweep            # the reference's table (bench/kernels.py) for 1..4096 tokens
+
+A step is one call of kernels.moe_layer (router GEMM, route, sort, two grouped projections,
+combine) on N tokens with every input already in HBM. The default workload is decode at 8
+tokens, the configuration the reference's headline is quoted on. The metric is the reference's
+(bench/kernels.py:52-55): bytes of expert weights of the experts that received a token, each
+counted once, over the layer time. Successive steps rotate through several layers' weights, as
+a decoder does, so that no step finds its weights in the 256 MB last-level cache.
+
+Prints ONE JSON line with the metric, a `roofline` object for the dominant kernel (the
+gate/up projection: two thirds of the weight bytes), timed per launch with events on the
+launch stream, and a `cpu_baseline` object: the per-expert PyTorch loop on this host's cores."""
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+import torch
+import torch.nn.functional as F
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+E, TOPK, H, I = 64, 8, 2048, 1024
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published
+EXPERT_BYTES = 3 * H * I * 2   # gate + up + down of one expert, fp16
+T4_WEIGHT_GBS_AT_8 = 232.98490131032196  # the reference's published figure for this metric (Tesla T4)
+
+# HBM bytes per launch of the gate/up projection from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
+# keyed by token count; filled from the summaries under profiles/ (None: not measured).
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def make_layers(n_layers, seed=0):
+    import cases
+
+    layers = []
+    for j in range(n_layers):
+        _, router, gu, dn = cases.layer(1, seed=seed + j)
+        layers.append((router, gu, dn))
+    return layers
+
+
+def hidden(N, seed=0):
+    return torch.randn(N, H, generator=torch.Generator().manual_seed(seed + 1000 + N)).half()
+
+
+def event_times(fn, reps):
+    """Per-call GPU time in ms, one event pair per call on the current stream."""
+    out = []
+    for _ in range(reps):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        b.synchronize()
+        out.append(a.elapsed_time(b))
+    return out
+
+
+def cpu_loop_baseline(h, router, gu, dn, used, reps=5):
+    """The reference per-expert loop (switchyard/moe.py:34-42) restated in oracle/, fp32, on the host."""
+    from oracle import moe_oracle as O
+
+    hf, rf, gf, df = h.float(), router.float(), gu.float(), dn.float()
+    idx, w = O.route(hf, rf, TOPK, False)
+    O.experts_loop(hf, idx, w, gf, df)
+    times = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        O.experts_loop(hf, idx, w, gf, df)
+        times.append(time.perf_counter() - t0)
+    t = statistics.median(times)
+    return {"value": used * EXPERT_BYTES / t / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"oracle per-expert loop, fp32 weights, {h.shape[0]} tokens, median of {reps} passes "
+                      f"({t * 1e3:.1f} ms each) after 1 warm-up; os.cpu_count()={os.cpu_count()}",
+            "us_per_layer": t * 1e6}
+
+
+def run_default(args):
+    from switchyard_amd import kernels
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    N = args.tokens
+    cpu_layers = make_layers(args.layers)
+    layers = [tuple(t.to(dev) for t in L) for L in cpu_layers]
+    h_cpu = hidden(N)
+    h = h_cpu.to(dev)
+    mode = args.mode
+
+    def step(j):
+        router, gu, dn = layers[j % len(layers)]
+        return kernels.moe_layer(h, router, gu, dn, TOPK, False, mode)
+
+    # experts that receive a token, per layer (the metric's numerator)
+    used = []
+    for router, gu, dn in layers:
+        idx, _ = kernels.route(h, router, TOPK, False)
+        used.append(int((torch.bincount(idx.flatten().long(), minlength=E) > 0).sum()))
+
+    for j in range(args.warmup):
+        step(j)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for j in range(args.steps):
+        step(j)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    used_mean = sum(used[j % len(layers)] for j in range(args.steps)) / args.steps
+    value = used_mean * EXPERT_BYTES / (ms_per_step / 1e3) / 1e9
+
+    # the same layer call timed with one event pair per call (the reference's method, median)
+    ev = event_times(lambda: step(0), 20)
+    ev_med = statistics.median(ev)
+
+    # dominant kernel: the gate/up projection, one event pair per launch on the launch stream
+    router, gu, dn = layers[0]
+    idx, w = kernels.route(h, router, TOPK, False)
+    counts, offsets, token, wsorted, pos_of = kernels.ext().sort_by_expert(idx, w, E)
+    M = idx.numel()
+    use_gemv = (mode if mode != "auto" else kernels._auto(N, M, E)) == "gemv"
+    rot = []
+    for r_, g_, d_ in layers:
+        i_, w_ = kernels.route(h, r_, TOPK, False)
+        s_ = kernels.ext().sort_by_expert(i_, w_, E)
+        rot.append((g_, s_[1], s_[2]))
+    calls = [0]
+
+    def gate_up():
+        g_, off_, tok_ = rot[calls[0] % len(rot)]
+        calls[0] += 1
+        if use_gemv:
+            return kernels.ext().grouped_gemv(h, tok_, g_, off_, M, True, None)
+        return kernels.ext().grouped_gemm(h, tok_, g_, off_, None, 0, M, True, None)
+
+    for _ in range(max(3, args.warmup)):
+        gate_up()
+    calls[0] = 0
+    kt = event_times(gate_up, max(args.steps, 20))
+    k_ms = sum(kt) / len(kt)
+    used_k = sum(used[j % len(layers)] for j in range(len(kt))) / len(kt)
+    if use_gemv or M // E < 300:
+        alg = used_k * 2 * H * I * 2                      # gate and up rows of every used expert, once
+        roof = {"bound": "hbm", "achieved": alg / (k_ms / 1e3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s"}
+    else:
+        alg = M * 4 * H * I                                # 2 * rows * 2I * H flops
+        roof = {"bound": "mfma", "achieved": alg / (k_ms / 1e3) / 1e12, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s"}
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(N)
+    roof["kernel"] = "gemv_kernel<swiglu> (gate/up projection)" if use_gemv else "gemm_kernel<swiglu> (gate/up projection)"
+    roof["us_per_launch"] = k_ms * 1e3
+    roof["algorithmic_per_launch"] = alg
+
+    cpu = cpu_loop_baseline(h_cpu, *cpu_layers[0], used[0])
+
+    line = {
+        "metric": "OLMoE MoE-layer expert-weight GB/s", "value": value, "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": value / T4_WEIGHT_GBS_AT_8 if N == 8 else None, "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": f"olmoe_moe_layer_{'decode' if N <= 64 else 'prefill'}_{N}tok", "tokens": N,
+                   "experts": E, "top_k": TOPK, "hidden": H, "expert_width": I, "mode": mode,
+                   "layers_rotated": len(layers), "experts_used_mean": used_mean},
+        "us_per_layer": ms_per_step * 1e3, "us_per_layer_event_median": ev_med * 1e3,
+        "frac_of_hbm_peak": value / HBM_PEAK_GBS,
+        "tflops": N * TOPK * 6 * H * I / (ms_per_step / 1e3) / 1e12,
+        "vs_baseline_note": "published figure is the reference's on one Tesla T4 (320 GB/s)",
+        "gpu": torch.cuda.get_device_name(0),
+        "roofline": roof, "cpu_baseline": cpu,
+    }
+    print(json.dumps(line), flush=True)
+
+
+def run_sweep(args):
+    """One JSON line per token count: the per-expert loop and the sorted loop in torch on the
+    GPU (the reference's columns), the kernels in auto / gemv / gemm, errors, GB/s and TFLOP/s."""
+    from oracle import moe_oracle as O
+    from switchyard_amd import kernels
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    layers = [tuple(t.to(dev) for t in L) for L in make_layers(args.layers)]
+    router, gu, dn = layers[0]
+    sizes = [int(x) for x in args.sweep.split(",")] if args.sweep != "all" else [1, 8, 16, 32, 64, 128, 256, 512, 1024, 2048, 4096]
+
+    def med(fn, reps=20, warm=3):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        return statistics.median(event_times(fn, reps))
+
+    print(json.dumps({"bench": "moe_layer_sweep", "gpu": torch.cuda.get_device_name(0), "experts": E, "top_k": TOPK,
+                      "hidden": H, "expert_width": I, "layers_rotated": len(layers)}), flush=True)
+    for N in sizes:
+        h = hidden(N).to(dev)
+        idx, w = O.route(h, router, TOPK, False)
+        j = [0]
+
+        def rotating(mode):
+            def fn():
+                r_, g_, d_ = layers[j[0] % len(layers)]
+                j[0] += 1
+                return kernels.moe_layer(h, r_, g_, d_, TOPK, False, mode)
+            return fn
+
+        rec = {"tokens": N}
+        rec["auto_ms"] = med(rotating("auto"))
+        rec["gemv_ms"] = med(rotating("gemv")) if N <= 1024 else None
+        rec["gemm_ms"] = med(rotating("gemm"))
+        if not args.no_loops:
+            rec["loop_ms"] = med(lambda: O.experts_loop(h, idx, w, gu, dn), reps=5, warm=1)
+            rec["sorted_loop_ms"] = med(lambda: O.experts_grouped(h, idx, w, gu, dn), reps=5, warm=1)
+        want = O.experts_loop(h.float(), idx, w.float(), gu.float(), dn.float())
+        rec["max_err_auto"] = (kernels.moe_layer(h, router, gu, dn, TOPK, False).float() - want).abs().max().item()
+        rec["max_err_fp16_loop"] = (O.experts_loop(h, idx, w, gu, dn).float() - want).abs().max().item()
+        cnt = torch.bincount(idx.flatten(), minlength=E)
+        used = int((cnt > 0).sum())
+        rec["max_rows_per_expert"], rec["experts_used"] = int(cnt.max()), used
+        best = min(x for x in (rec["auto_ms"], rec["gemv_ms"], rec["gemm_ms"]) if x)
+        rec["weight_GBps_auto"] = used * EXPERT_BYTES / (rec["auto_ms"] / 1e3) / 1e9
+        rec["weight_GBps_best"] = used * EXPERT_BYTES / (best / 1e3) / 1e9
+        rec["tflops_auto"] = N * TOPK * 6 * H * I / (rec["auto_ms"] / 1e3) / 1e12
+        rec["frac_hbm"] = rec["weight_GBps_auto"] / HBM_PEAK_GBS
+        rec["frac_mfma"] = rec["tflops_auto"] / MFMA_F16_PEAK_TFLOPS
+        print(json.dumps(rec), flush=True)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--tokens", type=int, default=8)
+    ap.add_argument("--mode", default="auto", choices=["auto", "gemv", "gemm"])
+    ap.add_argument("--layers", type=int, default=4, help="distinct layers' weights to rotate through")
+    ap.add_argument("--sweep", default=None, help='"all" or a comma list of token counts')
+    ap.add_argument("--no-loops", action="store_true", help="sweep: skip the torch per-expert loops")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this path runs on one GPU; --gpus must be 1 (no multi-GPU figure is produced)")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    with torch.no_grad():
+        if args.sweep:
+            run_sweep(args)
+        else:
+            run_default(args)
+
+
+if __name__ == "__main__":
+    main()

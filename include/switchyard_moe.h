@@ -1,0 +1,91 @@
+/* switchyard_moe.h: C ABI of libswitchyard_moe.so, the MI355X (gfx950) kernels of the OLMoE
+ * mixture-of-experts layer.
+ *
+ * Every entry point replaces one function of the reference's native module
+ * (switchyard/csrc/moe_kernels.cu, pybind surface at :491-500) and is what a binding for that
+ * path would call. Conventions:
+ *   - all pointers are device pointers on the current HIP device, borrowed for the call;
+ *     outputs (and workspaces) are allocated by the caller; nothing is allocated or freed here;
+ *   - `stream` is a hipStream_t passed as void*; work is enqueued on it and the call returns
+ *     without waiting;
+ *   - "f16" is IEEE binary16; every matrix is row-major and contiguous;
+ *   - the return value is 0 on success, otherwise an SY_ERR_* code, and sy_last_error()
+ *     returns a message for the calling thread;
+ *   - calls are re-entrant; the library keeps no state between calls.
+ */
+#ifndef SWITCHYARD_MOE_H
+#define SWITCHYARD_MOE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SY_API __attribute__((visibility("default")))
+
+#define SY_OK 0
+#define SY_ERR_ARG 1     /* an argument is out of the supported range */
+#define SY_ERR_LAUNCH 2  /* the HIP runtime refused a launch */
+
+#define SY_DTYPE_F16 0
+#define SY_DTYPE_F32 1
+
+/* Library version, major*10000 + minor*100 + patch. */
+SY_API int sy_version(void);
+
+/* Message of the last error on this thread ("" if none). */
+SY_API const char* sy_last_error(void);
+
+/* Replaces route() (moe_kernels.cu:73-89, kernel :23-71).
+ * logits [N,E] of `dtype` (SY_DTYPE_F16 or SY_DTYPE_F32) -> idx int32 [N,k], w [N,k] of the
+ * same dtype. Softmax in fp32; the k largest ordered by (logit descending, expert id
+ * ascending); w = p, or p / sum of the chosen k when norm != 0.
+ * Limits: 1 <= E <= 128, 1 <= k <= 8, k <= E (the reference's, :77). N == 0 is a no-op. */
+SY_API int sy_route(const void* logits, int dtype, int N, int E, int k, int norm, int32_t* idx, void* w, void* stream);
+
+/* Bytes of workspace sy_sort_by_expert needs for N*k choices (may be 0). */
+SY_API size_t sy_sort_workspace_bytes(int N, int k, int E);
+
+/* Replaces sort_by_expert() (moe_kernels.cu:142-157, kernels :112-139, plus the ATen
+ * cumsum/zeros/copy_ at :148-149, folded into the kernels).
+ * Stable counting sort of the flat choices i = t*k + s by idx[i], without atomics.
+ * idx int32 [N,k] with values in [0,E); w [N,k] of w_bytes (2 or 4) per element ->
+ * counts int32 [E], offsets int32 [E+1], token int32 [M], wsorted [M], pos_of int32 [M],
+ * M = N*k. `workspace` holds sy_sort_workspace_bytes() bytes. Choices whose id is outside
+ * [0,E) are ignored (they get no row). Limits: 1 <= E <= 512. */
+SY_API int sy_sort_by_expert(const int32_t* idx, const void* w, int w_bytes, int N, int k, int E, int32_t* counts,
+                      int32_t* offsets, int32_t* token, void* wsorted, int32_t* pos_of, void* workspace,
+                      size_t workspace_bytes, void* stream);
+
+/* Replaces grouped_gemv() (moe_kernels.cu:385-415, kernel :308-383): the decode weight stream.
+ * For every expert e and row r in offsets[e]..offsets[e+1]:
+ *   C[r,:] = epilogue(A[a_rows ? a_rows[r] : r, :] @ B[e]^T)
+ * A f16 [*,K]; a_rows int32 [rows] or NULL; B f16 [E,Nfull,K] (nn.Linear layout),
+ * Nfull = 2*Nout when swiglu (gate rows first) else Nout; offsets int32 [E+1];
+ * scale f16 [rows] or NULL; C f16 [rows,Nout].
+ * swiglu: C = f16(f16(silu(f16(gate))) * f16(up)); scale: C = f16(f16(acc) * scale[r]).
+ * Limits: K % 8 == 0, K <= 8192. rows == 0 is a no-op. */
+SY_API int sy_grouped_gemv(const void* A, const int32_t* a_rows, const void* B, const int32_t* offsets, int E, int rows,
+                    int Nout, int K, int swiglu, const void* scale, void* C, void* stream);
+
+/* Replaces grouped_gemm() (moe_kernels.cu:264-298, kernel :167-261): the same function on
+ * MFMA tiles for many rows per expert. The row tiles of every expert are derived from
+ * `offsets` inside the kernel, so the reference's tile_offsets / total_tiles arguments (and
+ * the host read behind them, kernels.py:61) have no counterpart here.
+ * Limits: K % 32 == 0. rows == 0 is a no-op. */
+SY_API int sy_grouped_gemm(const void* A, const int32_t* a_rows, const void* B, const int32_t* offsets, int E, int rows,
+                    int Nout, int K, int swiglu, const void* scale, void* C, void* stream);
+
+/* Replaces combine() (moe_kernels.cu:435-444, kernel :419-433).
+ * out[t,:] = f16(sum over t's k choices, in ascending expert id, of y[pos_of[t*k+j],:]) with
+ * the sum in fp32. y f16 [M,H]; pos_of int32 [N*k]; idx int32 [N,k]; out f16 [N,H].
+ * Limits: H % 8 == 0, 1 <= k <= 64. N == 0 is a no-op. */
+SY_API int sy_combine(const void* y, const int32_t* pos_of, const int32_t* idx, int N, int k, int H, void* out,
+               void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SWITCHYARD_MOE_H */

@@ -1,0 +1,153 @@
+"""ctypes binding of libswitchyard_moe.so (C ABI in include/switchyard_moe.h).
+
+`Ext` offers the functions of the reference's pybind module `switchyard_moe`
+(switchyard/csrc/moe_kernels.cu:491-500) with the same names, argument order and results,
+so code written against `kernels.ext()` keeps working. Outputs are allocated here with
+torch.empty on the current stream; the library itself never allocates. ctypes releases the
+GIL around every call, as the reference's call guards do.
+
+There is no fallback: if the library is missing and cannot be built, loading raises."""
+
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libswitchyard_moe.so")
+
+_c_int, _c_void_p, _c_size_t = ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t
+
+# name -> (restype, argtypes); mirrors include/switchyard_moe.h
+SIGNATURES = {
+    "sy_version": (_c_int, []),
+    "sy_last_error": (ctypes.c_char_p, []),
+    "sy_route": (_c_int, [_c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p]),
+    "sy_sort_workspace_bytes": (_c_size_t, [_c_int, _c_int, _c_int]),
+    "sy_sort_by_expert": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p,
+                                   _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_size_t, _c_void_p]),
+    "sy_grouped_gemv": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int,
+                                 _c_void_p, _c_void_p, _c_void_p]),
+    "sy_grouped_gemm": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int,
+                                 _c_void_p, _c_void_p, _c_void_p]),
+    "sy_combine": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p]),
+}
+
+
+def load_library(path=LIB_PATH):
+    """dlopen the library and declare every entry point; builds it first if it is absent."""
+    if not os.path.exists(path):
+        from . import build
+
+        try:
+            build.build()
+        except Exception as exc:  # no hipcc, or the compile failed
+            raise RuntimeError(f"switchyard_amd: {path} is missing and could not be built: {exc}") from exc
+    lib = ctypes.CDLL(path)
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the library does not export it
+        fn.restype, fn.argtypes = restype, argtypes
+    return lib
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _check(t, name, dtype=None):
+    if not (t.is_cuda and t.is_contiguous()):
+        raise RuntimeError(f"{name} must be a contiguous GPU tensor")
+    if dtype is not None and t.dtype != dtype:
+        raise RuntimeError(f"{name} must be {dtype}, got {t.dtype}")
+
+
+_DTYPE_CODE = {torch.float16: 0, torch.float32: 1}
+
+
+class Ext:
+    """The native module: route, sort_by_expert, grouped_gemv, grouped_gemm, combine."""
+
+    def __init__(self, lib=None):
+        self.lib = lib or load_library()
+
+    def _call(self, fn, *args):
+        rc = fn(*args)
+        if rc:
+            raise RuntimeError(self.lib.sy_last_error().decode())
+
+    def version(self):
+        return self.lib.sy_version()
+
+    def route(self, logits, k, norm):
+        """logits [N, E] f16 (or f32) -> [idx int32 [N, k], w [N, k] in logits' dtype]."""
+        _check(logits, "logits")
+        if logits.dtype not in _DTYPE_CODE:
+            raise RuntimeError("route: fp16 logits")
+        N, E = logits.shape
+        idx = torch.empty((N, k), dtype=torch.int32, device=logits.device)
+        w = torch.empty((N, k), dtype=logits.dtype, device=logits.device)
+        self._call(self.lib.sy_route, logits.data_ptr(), _DTYPE_CODE[logits.dtype], N, E, int(k), int(bool(norm)),
+                   idx.data_ptr(), w.data_ptr(), _stream())
+        return [idx, w]
+
+    def sort_by_expert(self, idx, w, E):
+        """idx int32 [N, k], w [N, k] -> [counts [E], offsets [E+1], token [M], wsorted [M], pos_of [M]]."""
+        _check(idx, "idx", torch.int32)
+        _check(w, "w")
+        N, k = idx.shape
+        M, dev = N * k, idx.device
+        counts = torch.empty(E, dtype=torch.int32, device=dev)
+        offsets = torch.empty(E + 1, dtype=torch.int32, device=dev)
+        token = torch.empty(M, dtype=torch.int32, device=dev)
+        wsorted = torch.empty(M, dtype=w.dtype, device=dev)
+        pos_of = torch.empty(M, dtype=torch.int32, device=dev)
+        need = self.lib.sy_sort_workspace_bytes(N, k, E)
+        ws = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
+        self._call(self.lib.sy_sort_by_expert, idx.data_ptr(), w.data_ptr(), w.element_size(), N, k, int(E),
+                   counts.data_ptr(), offsets.data_ptr(), token.data_ptr(), wsorted.data_ptr(), pos_of.data_ptr(),
+                   ws.data_ptr() if need else None, need, _stream())
+        return [counts, offsets, token, wsorted, pos_of]
+
+    def _grouped(self, fn, A, a_rows, B, offsets, rows, swiglu, scale):
+        _check(A, "A", torch.float16)
+        _check(B, "B", torch.float16)
+        _check(offsets, "offsets", torch.int32)
+        if a_rows is not None:
+            _check(a_rows, "a_rows", torch.int32)
+        if scale is not None:
+            _check(scale, "scale", torch.float16)
+        E, Nfull, K = B.shape
+        if A.shape[1] != K:
+            raise RuntimeError("grouped: K must match")
+        if offsets.numel() != E + 1:
+            raise RuntimeError("grouped: offsets must have E + 1 entries")
+        if a_rows is not None and a_rows.numel() < rows or scale is not None and scale.numel() < rows:
+            raise RuntimeError("grouped: a_rows / scale shorter than rows")
+        if a_rows is None and A.shape[0] < rows:
+            raise RuntimeError("grouped: A has fewer rows than `rows`")
+        Nout = Nfull // 2 if swiglu else Nfull
+        C = torch.empty((rows, Nout), dtype=A.dtype, device=A.device)
+        self._call(fn, A.data_ptr(), a_rows.data_ptr() if a_rows is not None else None, B.data_ptr(),
+                   offsets.data_ptr(), E, int(rows), Nout, K, int(bool(swiglu)),
+                   scale.data_ptr() if scale is not None else None, C.data_ptr(), _stream())
+        return C
+
+    def grouped_gemv(self, A, a_rows, B, offsets, rows, swiglu, scale):
+        return self._grouped(self.lib.sy_grouped_gemv, A, a_rows, B, offsets, rows, swiglu, scale)
+
+    def grouped_gemm(self, A, a_rows, B, offsets, tile_offsets, total_tiles, rows, swiglu, scale):
+        """tile_offsets / total_tiles are accepted for the reference's call shape and unused:
+        the kernel derives its row tiles from `offsets`."""
+        return self._grouped(self.lib.sy_grouped_gemm, A, a_rows, B, offsets, rows, swiglu, scale)
+
+    def combine(self, y, pos_of, idx, n_tokens):
+        _check(y, "y", torch.float16)
+        _check(pos_of, "pos_of", torch.int32)
+        _check(idx, "idx", torch.int32)
+        H, k = y.shape[1], idx.shape[1]
+        if pos_of.numel() < n_tokens * k or idx.shape[0] < n_tokens:
+            raise RuntimeError("combine: pos_of / idx shorter than n_tokens * k")
+        out = torch.empty((n_tokens, H), dtype=y.dtype, device=y.device)
+        self._call(self.lib.sy_combine, y.data_ptr(), pos_of.data_ptr(), idx.data_ptr(), int(n_tokens), k, H,
+                   out.data_ptr(), _stream())
+        return out

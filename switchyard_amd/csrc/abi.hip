@@ -1,0 +1,27 @@
+// Error plumbing and version of the C ABI (include/switchyard_moe.h).
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "common.h"
+
+namespace {
+thread_local char g_error[512] = "";
+}
+
+int sy_fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int sy_check_launch(const char* what) {
+  const hipError_t err = hipGetLastError();
+  if (err == hipSuccess) return SY_OK;
+  return sy_fail(SY_ERR_LAUNCH, "%s: launch failed: %s", what, hipGetErrorString(err));
+}
+
+extern "C" SY_API int sy_version(void) { return 100; }
+
+extern "C" SY_API const char* sy_last_error(void) { return g_error; }

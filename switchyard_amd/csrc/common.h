@@ -1,0 +1,61 @@
+// Shared device helpers for the gfx950 MoE kernels: 16-bit float vectors, wavefront-64
+// reductions (DPP inside a row of 16 lanes, cross-lane shuffles above that) and the
+// error plumbing of the C ABI.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/switchyard_moe.h"
+
+typedef _Float16 half_t;
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+constexpr int WAVE = 64;
+
+// Records a message for sy_last_error() and returns `code`.
+int sy_fail(int code, const char* fmt, ...);
+// Returns SY_OK, or records the pending HIP launch error and returns SY_ERR_LAUNCH.
+int sy_check_launch(const char* what);
+
+#define SY_REQUIRE(cond, ...) \
+  do {                        \
+    if (!(cond)) return sy_fail(SY_ERR_ARG, __VA_ARGS__); \
+  } while (0)
+
+// ---- DPP: rotate right by N inside each row of 16 lanes (row_ror:N = 0x120 + N).
+template <int N>
+__device__ __forceinline__ int dpp_row_ror(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, 0x120 + N, 0xf, 0xf, false);
+}
+template <int N>
+__device__ __forceinline__ float dpp_row_ror(float v) {
+  return __int_as_float(dpp_row_ror<N>(__float_as_int(v)));
+}
+
+// All-reduce over the 64 lanes of a wavefront; every lane ends with the same bits because
+// each step combines two values that are themselves identical across the partner lanes.
+template <typename T, typename Op>
+__device__ __forceinline__ T wave_allreduce(T v, Op op) {
+  v = op(v, dpp_row_ror<8>(v));
+  v = op(v, dpp_row_ror<4>(v));
+  v = op(v, dpp_row_ror<2>(v));
+  v = op(v, dpp_row_ror<1>(v));
+  v = op(v, __shfl_xor(v, 16, WAVE));
+  v = op(v, __shfl_xor(v, 32, WAVE));
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+  return wave_allreduce(v, [](float a, float b) { return fmaxf(a, b); });
+}
+__device__ __forceinline__ float wave_sum(float v) {
+  return wave_allreduce(v, [](float a, float b) { return a + b; });
+}
+
+__device__ __forceinline__ uint64_t lanemask_lt() {
+  return (1ull << (threadIdx.x & 63)) - 1ull;
+}

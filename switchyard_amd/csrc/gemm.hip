@@ -1,0 +1,234 @@
+// grouped_gemm: the prefill path. Every expert's slice of the sorted rows goes through that
+// expert's weights on fp16 MFMA tiles, all experts in one launch.
+//
+// Tile: 128 rows x 256 weight rows, K in slices of 32, 4 wavefronts (2 x 2), each computing
+// 64 rows x 128 weight rows as 2 x 4 v_mfma_f32_32x32x16_f16 blocks with fp32 accumulators.
+// With SwiGLU the 256 weight rows are 128 gate rows and the 128 up rows of the same output
+// columns, and a wavefront holds gate and up of the same 64 columns, so the activation is
+// applied in registers. Weights are the MFMA M operand and rows the N operand: a lane ends
+// up with runs of 4 consecutive output columns of one row and stores them as 8 bytes.
+//
+// Rows are gathered from the unsorted input inside the kernel (a_rows). K-slices are
+// double-buffered in LDS: while the MFMAs consume slice i from one buffer, the global loads
+// of slice i+1 are in flight into registers and are written to the other buffer afterwards,
+// one barrier per slice. LDS rows are padded to 80 bytes so that the 128-bit operand reads
+// of 16 consecutive lanes fall in distinct banks.
+//
+// The row tiles of all experts are laid end to end. The map from a tile to (expert, first
+// row) is rebuilt by every workgroup from `offsets` with one wavefront scan, so the host
+// needs neither the reference's tile_offsets tensor nor a device-to-host read; the grid is
+// sized for the worst case and surplus workgroups leave at once. Workgroups are renumbered
+// so that consecutive tiles, which share rows or weights, run on the same XCD and meet in
+// its L2.
+//
+// Replaces grouped_gemm_kernel / grouped_gemm of the reference
+// (switchyard/csrc/moe_kernels.cu:159-298); epilogue rounding points as :253-259.
+#include "common.h"
+
+namespace {
+
+constexpr int BM = 128;          // rows per tile
+constexpr int BW = 256;          // weight rows per tile
+constexpr int BK = 32;           // K per slice
+constexpr int LDS_LD = BK + 8;   // halves per LDS row (80 bytes)
+constexpr int GEMM_THREADS = 256;
+constexpr int XCDS = 8;
+
+__device__ __forceinline__ half_t swiglu_f16(float gate, float up) {
+  const float g = (float)(half_t)gate, u = (float)(half_t)up;
+  const float s = (float)(half_t)(g / (1.f + expf(-g)));
+  return (half_t)(s * u);
+}
+
+template <bool SWIGLU, bool SCALE>
+__global__ void __launch_bounds__(GEMM_THREADS, 2)
+gemm_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const half_t* __restrict__ B,
+            const int* __restrict__ offsets, int E, int Nout, int K, const half_t* __restrict__ scale,
+            half_t* __restrict__ C, int ncol_tiles, int per_xcd) {
+  __shared__ __attribute__((aligned(16))) half_t lds[2][(BM + BW) * LDS_LD];
+  __shared__ int s_tile[3];
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+
+  // consecutive logical tiles on one XCD (workgroups are dealt round-robin to the XCDs)
+  const int logical = (blockIdx.x % XCDS) * per_xcd + blockIdx.x / XCDS;
+  const int row_tile = logical / ncol_tiles, col_tile = logical % ncol_tiles;
+
+  if (tid == 0) s_tile[0] = -1;
+  __syncthreads();
+  if (wave == 0) {
+    int run = 0;
+    for (int e0 = 0; e0 < E; e0 += WAVE) {
+      const int e = e0 + lane;
+      const int first = e < E ? offsets[e] : 0, last = e < E ? offsets[e + 1] : 0;
+      const int tiles = (last - first + BM - 1) / BM;
+      int inc = tiles;
+      for (int o = 1; o < WAVE; o <<= 1) {
+        const int up = __shfl_up(inc, o, WAVE);
+        if (lane >= o) inc += up;
+      }
+      const int lo = run + inc - tiles;
+      if (row_tile >= lo && row_tile < lo + tiles) {
+        s_tile[0] = e;
+        s_tile[1] = first + (row_tile - lo) * BM;
+        s_tile[2] = last;
+      }
+      run += __shfl(inc, WAVE - 1, WAVE);
+    }
+  }
+  __syncthreads();
+  const int e = s_tile[0];
+  if (e < 0) return;
+  const int row0 = s_tile[1], row_end = s_tile[2];
+  const int nrows = min(BM, row_end - row0);
+
+  constexpr int COLS = SWIGLU ? BW / 2 : BW;  // output columns per tile
+  const int n0 = col_tile * COLS;
+  const int Nfull = SWIGLU ? 2 * Nout : Nout;
+  const half_t* Be = B + (size_t)e * Nfull * K;
+
+  // ---- loader: thread t moves 16-byte chunk (t & 3) of rows (t >> 2) + 64*q
+  const int lrow = tid >> 2, lch = (tid & 3) * 8;
+  const half_t* pa[2];
+  const half_t* pb[4];
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+    const int r = lrow + 64 * q;
+    pa[q] = r < nrows ? A + (size_t)(a_rows ? a_rows[row0 + r] : row0 + r) * K + lch : nullptr;
+  }
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int br = lrow + 64 * q;
+    int wr, col;
+    if (SWIGLU) {
+      col = n0 + (br & (COLS - 1));
+      wr = br < COLS ? col : Nout + col;
+    } else {
+      col = n0 + br;
+      wr = col;
+    }
+    pb[q] = col < Nout ? Be + (size_t)wr * K + lch : nullptr;
+  }
+  const half8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  half8_t ra[2], rb[4];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int q = 0; q < 2; ++q) ra[q] = pa[q] ? *reinterpret_cast<const half8_t*>(pa[q] + k0) : zero8;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) rb[q] = pb[q] ? *reinterpret_cast<const half8_t*>(pb[q] + k0) : zero8;
+  };
+  auto stash = [&](int buf) {
+    half_t* as = lds[buf];
+    half_t* bs = as + BM * LDS_LD;
+#pragma unroll
+    for (int q = 0; q < 2; ++q) *reinterpret_cast<half8_t*>(as + (lrow + 64 * q) * LDS_LD + lch) = ra[q];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) *reinterpret_cast<half8_t*>(bs + (lrow + 64 * q) * LDS_LD + lch) = rb[q];
+  };
+
+  // ---- wavefront tile
+  const int wm = wave >> 1, wn = wave & 1;
+  const int l32 = lane & 31, lk = (lane >> 5) * 8;
+  int brow[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) brow[j] = SWIGLU ? (j >> 1) * COLS + wn * 64 + (j & 1) * 32 : wn * 128 + j * 32;
+
+  float16_t acc[2][4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  fetch(0);
+  stash(0);
+  __syncthreads();
+  const int nk = K / BK;
+  for (int kt = 0; kt < nk; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < nk) fetch((kt + 1) * BK);
+    const half_t* as = lds[buf] + (wm * 64 + l32) * LDS_LD + lk;
+    const half_t* bs = lds[buf] + (BM + l32) * LDS_LD + lk;
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += 16) {
+      half8_t xf[2], wf[4];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) xf[i] = *reinterpret_cast<const half8_t*>(as + i * 32 * LDS_LD + kk);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) wf[j] = *reinterpret_cast<const half8_t*>(bs + brow[j] * LDS_LD + kk);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[j], xf[i], acc[i][j], 0, 0, 0);
+    }
+    if (kt + 1 < nk) stash(buf ^ 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue: acc element 4*q + r of block (i, j) is row i*32 + l32, column 8*q + 4*(lane/32) + r
+  const int chalf = (lane >> 5) * 4;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int row = row0 + wm * 64 + i * 32 + l32;
+    if (row >= row_end) continue;
+    const float sc_row = SCALE ? (float)scale[row] : 1.f;
+    half_t* crow = C + (size_t)row * Nout;
+    constexpr int NJ = SWIGLU ? 2 : 4;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const int cbase = n0 + (SWIGLU ? wn * 64 + j * 32 : wn * 128 + j * 32) + chalf;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int c0 = cbase + 8 * q;
+        half4_t o;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float v = acc[i][j][4 * q + r];
+          if (SWIGLU) o[r] = swiglu_f16(v, acc[i][j + 2][4 * q + r]);
+          else if (SCALE) o[r] = (half_t)((float)(half_t)v * sc_row);
+          else o[r] = (half_t)v;
+        }
+        if (c0 + 3 < Nout && (Nout & 3) == 0) {
+          *reinterpret_cast<half4_t*>(crow + c0) = o;
+        } else {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (c0 + r < Nout) crow[c0 + r] = o[r];
+        }
+      }
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" SY_API int sy_grouped_gemm(const void* A, const int32_t* a_rows, const void* B, const int32_t* offsets, int E,
+                               int rows, int Nout, int K, int swiglu, const void* scale, void* C, void* stream) {
+  SY_REQUIRE(rows >= 0 && E >= 1 && Nout >= 1, "grouped_gemm: rows = %d, E = %d, Nout = %d", rows, E, Nout);
+  SY_REQUIRE(K >= BK && K % BK == 0, "grouped_gemm: K must be a multiple of %d (got %d)", BK, K);
+  SY_REQUIRE(!(swiglu && scale), "grouped_gemm: swiglu and scale are not combined");
+  if (rows == 0) return SY_OK;
+  SY_REQUIRE(A && B && offsets && C, "grouped_gemm: null pointer");
+  const int cols = swiglu ? BW / 2 : BW;
+  const int ncol_tiles = (Nout + cols - 1) / cols;
+  // sum over experts of ceil(count / BM) <= rows / BM + (experts with rows) <= rows / BM + min(E, rows)
+  const long max_row_tiles = rows / BM + (E < rows ? E : rows);
+  const long total = max_row_tiles * ncol_tiles;
+  SY_REQUIRE(total < (1l << 31) - XCDS, "grouped_gemm: too many tiles");
+  const int per_xcd = (int)((total + XCDS - 1) / XCDS);
+  const int grid = per_xcd * XCDS;
+  hipStream_t st = (hipStream_t)stream;
+  const half_t* a = (const half_t*)A;
+  const half_t* b = (const half_t*)B;
+  const half_t* s = (const half_t*)scale;
+  half_t* c = (half_t*)C;
+  if (swiglu)
+    gemm_kernel<true, false><<<grid, GEMM_THREADS, 0, st>>>(a, a_rows, b, offsets, E, Nout, K, nullptr, c, ncol_tiles, per_xcd);
+  else if (s)
+    gemm_kernel<false, true><<<grid, GEMM_THREADS, 0, st>>>(a, a_rows, b, offsets, E, Nout, K, s, c, ncol_tiles, per_xcd);
+  else
+    gemm_kernel<false, false><<<grid, GEMM_THREADS, 0, st>>>(a, a_rows, b, offsets, E, Nout, K, nullptr, c, ncol_tiles, per_xcd);
+  return sy_check_launch("grouped_gemm");
+}

@@ -1,0 +1,273 @@
+// sort_by_expert: stable counting sort of the N*k routing choices by expert id, without
+// atomics, so a run is deterministic.
+//
+// The flat choices i = t*k + s are cut into consecutive pieces, one per wavefront. A
+// wavefront walks its piece 64 choices at a time. For one group of 64 it finds, for every
+// lane, the set of lanes holding the same expert (a "match" built from one ballot per bit of
+// the expert id); the number of matching lanes below a lane is that choice's rank inside the
+// group, and the highest matching lane adds the group's count to the wavefront's running
+// per-expert counter in LDS (one writer per expert, so no atomic is needed).
+//
+//   pass 1  per-wavefront histograms
+//   scan    per expert: exclusive prefix over wavefronts (stability across pieces) and the
+//           total; then an exclusive scan over experts gives `offsets`
+//   pass 2  the same walk again; row = offsets[e] + prefix[wavefront][e] + running + rank
+//
+// Up to SMALL_M choices the three steps run in one launch of one workgroup (decode: one
+// launch instead of the reference's two kernels and three library calls). Above that, pass 1
+// is a launch over many workgroups that leaves its histograms in the workspace, and the
+// second launch does the scan redundantly in every workgroup before its pass 2.
+//
+// Replaces count_kernel / assign_kernel / sort_by_expert of the reference
+// (switchyard/csrc/moe_kernels.cu:91-157).
+#include "common.h"
+
+namespace {
+
+constexpr int SORT_THREADS = 1024;
+constexpr int SORT_WAVES = SORT_THREADS / WAVE;  // 16
+constexpr int SMALL_M = 8192;                    // one workgroup sorts up to this many choices
+constexpr int PIECE = 512;                       // choices per wavefront in the large path
+constexpr int MAX_E = 512;                     // keeps every launch under 64 KB of LDS
+
+// Lanes of this wavefront whose key equals mine (restricted to `valid` lanes).
+__device__ __forceinline__ uint64_t match_lanes(int key, bool valid, int nbits) {
+  uint64_t m = __ballot(valid);
+  for (int b = 0; b < nbits; ++b) {
+    const bool bit = (key >> b) & 1;
+    const uint64_t bal = __ballot(bit);
+    m &= bit ? bal : ~bal;
+  }
+  return m;
+}
+
+// Pass 1 for one wavefront: hist[e] += number of choices in [lo, hi) equal to e.
+__device__ __forceinline__ void count_piece(const int* __restrict__ idx, int lo, int hi, int E, int nbits, int* hist) {
+  const int lane = threadIdx.x & 63;
+  for (int base = lo; base < hi; base += WAVE) {
+    const int i = base + lane;
+    int key = i < hi ? idx[i] : -1;
+    const bool valid = (unsigned)key < (unsigned)E;  // ids outside [0, E) are ignored
+    key = valid ? key : 0;
+    const uint64_t m = match_lanes(key, valid, nbits);
+    const int rank = __popcll(m & lanemask_lt()), cnt = __popcll(m);
+    if (valid && rank == cnt - 1) hist[key] += cnt;  // one lane per expert
+  }
+}
+
+// Pass 2 for one wavefront: base[e] is the row of this wavefront's first choice of expert e.
+template <typename W>
+__device__ __forceinline__ void assign_piece(const int* __restrict__ idx, const W* __restrict__ w, int lo, int hi, int k,
+                                             int E, int nbits, int* base, int* __restrict__ token, W* __restrict__ wsorted,
+                                             int* __restrict__ pos_of) {
+  const int lane = threadIdx.x & 63;
+  for (int at = lo; at < hi; at += WAVE) {
+    const int i = at + lane;
+    int key = i < hi ? idx[i] : -1;
+    const bool valid = (unsigned)key < (unsigned)E;
+    key = valid ? key : 0;
+    const uint64_t m = match_lanes(key, valid, nbits);
+    const int rank = __popcll(m & lanemask_lt()), cnt = __popcll(m);
+    int row = 0;
+    if (valid) row = base[key] + rank;
+    // every lane has read base[] before the one writer per expert updates it
+    __builtin_amdgcn_wave_barrier();
+    if (valid) {
+      token[row] = i / k;
+      wsorted[row] = w[i];
+      pos_of[i] = row;
+      if (rank == cnt - 1) base[key] += cnt;
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+// Exclusive scan over experts of total[0..E) into offs[0..E], E <= 1024, by the whole
+// workgroup (SORT_THREADS threads). tmp holds SORT_WAVES ints.
+__device__ __forceinline__ void scan_experts(const int* total, int E, int* offs, int* tmp) {
+  const int t = threadIdx.x, lane = t & 63, wv = t >> 6;
+  const int v = t < E ? total[t] : 0;
+  int inc = v;
+  for (int o = 1; o < WAVE; o <<= 1) {
+    const int up = __shfl_up(inc, o, WAVE);
+    if (lane >= o) inc += up;
+  }
+  if (lane == WAVE - 1) tmp[wv] = inc;
+  __syncthreads();
+  int before = 0;
+  for (int j = 0; j < wv; ++j) before += tmp[j];
+  if (t < E) offs[t] = before + inc - v;
+  if (t == E - 1) offs[E] = before + inc;
+  __syncthreads();
+}
+
+// ---------------------------------------------------------------- one workgroup does it all
+template <typename W>
+__global__ void __launch_bounds__(SORT_THREADS)
+sort_small_kernel(const int* __restrict__ idx, const W* __restrict__ w, int M, int k, int E, int nbits,
+                  int* __restrict__ counts, int* __restrict__ offsets, int* __restrict__ token,
+                  W* __restrict__ wsorted, int* __restrict__ pos_of) {
+  extern __shared__ int lds[];
+  int* hist = lds;                     // [SORT_WAVES][E]
+  int* total = hist + SORT_WAVES * E;  // [E]
+  int* offs = total + E;               // [E+1]
+  int* tmp = offs + E + 1;             // [SORT_WAVES]
+  const int t = threadIdx.x, wv = t >> 6;
+  for (int j = t; j < SORT_WAVES * E; j += SORT_THREADS) hist[j] = 0;
+  __syncthreads();
+
+  const int piece = ((M + SORT_WAVES - 1) / SORT_WAVES + WAVE - 1) / WAVE * WAVE;
+  const int lo = min(wv * piece, M), hi = min(lo + piece, M);
+  count_piece(idx, lo, hi, E, nbits, hist + wv * E);
+  __syncthreads();
+
+  if (t < E) {
+    int run = 0;
+    for (int j = 0; j < SORT_WAVES; ++j) {
+      const int c = hist[j * E + t];
+      hist[j * E + t] = run;
+      run += c;
+    }
+    total[t] = run;
+    counts[t] = run;
+  }
+  __syncthreads();
+  scan_experts(total, E, offs, tmp);
+  for (int j = t; j <= E; j += SORT_THREADS) offsets[j] = offs[j];
+  for (int j = t; j < SORT_WAVES * E; j += SORT_THREADS) hist[j] += offs[j % E];
+  __syncthreads();
+
+  assign_piece(idx, w, lo, hi, k, E, nbits, hist + wv * E, token, wsorted, pos_of);
+}
+
+// ---------------------------------------------------------------- many workgroups
+// Launch 1: virtual wavefront v = blockIdx.x * SORT_WAVES + wave owns choices
+// [v*PIECE, (v+1)*PIECE) and writes its histogram to ws[v][0..E).
+__global__ void __launch_bounds__(SORT_THREADS)
+sort_count_kernel(const int* __restrict__ idx, int M, int E, int nbits, int* __restrict__ ws) {
+  extern __shared__ int lds[];  // [SORT_WAVES][E]
+  const int t = threadIdx.x, wv = t >> 6;
+  for (int j = t; j < SORT_WAVES * E; j += SORT_THREADS) lds[j] = 0;
+  __syncthreads();
+  const int v = blockIdx.x * SORT_WAVES + wv;
+  const long lo64 = (long)v * PIECE;
+  const int lo = (int)(lo64 < M ? lo64 : M), hi = min(lo + PIECE, M);
+  count_piece(idx, lo, hi, E, nbits, lds + wv * E);
+  __syncthreads();
+  int* out = ws + (size_t)blockIdx.x * SORT_WAVES * E;
+  for (int j = t; j < SORT_WAVES * E; j += SORT_THREADS) out[j] = lds[j];
+}
+
+// Launch 2: every workgroup sums the histograms of all virtual wavefronts before its own
+// (and of all of them, for the totals), scans, and assigns its pieces.
+template <typename W>
+__global__ void __launch_bounds__(SORT_THREADS)
+sort_assign_kernel(const int* __restrict__ idx, const W* __restrict__ w, int M, int k, int E, int nbits,
+                   const int* __restrict__ ws, int nvirtual, int* __restrict__ counts, int* __restrict__ offsets,
+                   int* __restrict__ token, W* __restrict__ wsorted, int* __restrict__ pos_of) {
+  extern __shared__ int lds[];
+  int* base = lds;                         // [SORT_WAVES][E]
+  int* part_before = base + SORT_WAVES * E;  // [parts][E]
+  int* part_total = part_before + SORT_THREADS;
+  int* total = part_total + SORT_THREADS;  // [E]
+  int* before = total + E;                 // [E]
+  int* offs = before + E;                  // [E+1]
+  int* tmp = offs + E + 1;                 // [SORT_WAVES]
+  const int t = threadIdx.x, wv = t >> 6;
+  const int v0 = blockIdx.x * SORT_WAVES;
+
+  // thread (part, e): sums ws[v][e] over v = part, part + parts, ...
+  const int parts = SORT_THREADS / E;  // >= 1 because E <= 1024
+  const int e = t % E, part = t / E;
+  int sb = 0, st = 0;
+  if (part < parts) {
+    for (int v = part; v < nvirtual; v += parts) {
+      const int c = ws[(size_t)v * E + e];
+      st += c;
+      if (v < v0) sb += c;
+    }
+    part_before[part * E + e] = sb;
+    part_total[part * E + e] = st;
+  }
+  __syncthreads();
+  if (t < E) {
+    int b = 0, s = 0;
+    for (int j = 0; j < parts; ++j) {
+      b += part_before[j * E + t];
+      s += part_total[j * E + t];
+    }
+    before[t] = b;
+    total[t] = s;
+    if (blockIdx.x == 0) counts[t] = s;
+  }
+  __syncthreads();
+  scan_experts(total, E, offs, tmp);
+  if (blockIdx.x == 0)
+    for (int j = t; j <= E; j += SORT_THREADS) offsets[j] = offs[j];
+  if (t < E) {
+    int run = offs[t] + before[t];
+    for (int j = 0; j < SORT_WAVES; ++j) {
+      base[j * E + t] = run;
+      if (v0 + j < nvirtual) run += ws[(size_t)(v0 + j) * E + t];
+    }
+  }
+  __syncthreads();
+  const long lo64 = (long)(v0 + wv) * PIECE;
+  const int lo = (int)(lo64 < M ? lo64 : M), hi = min(lo + PIECE, M);
+  assign_piece(idx, w, lo, hi, k, E, nbits, base + wv * E, token, wsorted, pos_of);
+}
+
+int bits_for(int E) {
+  int b = 0;
+  while ((1 << b) < E) ++b;
+  return b;
+}
+
+int large_blocks(long M) { return (int)((M + (long)PIECE * SORT_WAVES - 1) / ((long)PIECE * SORT_WAVES)); }
+
+template <typename W>
+int launch_sort(const int32_t* idx, const void* w, int M, int k, int E, int32_t* counts, int32_t* offsets,
+                int32_t* token, void* wsorted, int32_t* pos_of, void* workspace, hipStream_t stream) {
+  const int nbits = bits_for(E);
+  if (M <= SMALL_M) {
+    const size_t lds = sizeof(int) * ((size_t)SORT_WAVES * E + 2 * E + 1 + SORT_WAVES);
+    sort_small_kernel<W><<<1, SORT_THREADS, lds, stream>>>(idx, (const W*)w, M, k, E, nbits, counts, offsets, token,
+                                                           (W*)wsorted, pos_of);
+    return sy_check_launch("sort_by_expert");
+  }
+  const int blocks = large_blocks(M), nvirtual = blocks * SORT_WAVES;
+  sort_count_kernel<<<blocks, SORT_THREADS, sizeof(int) * SORT_WAVES * E, stream>>>(idx, M, E, nbits, (int*)workspace);
+  if (int rc = sy_check_launch("sort_by_expert (count)")) return rc;
+  const size_t lds = sizeof(int) * ((size_t)SORT_WAVES * E + 2 * SORT_THREADS + 3 * E + 1 + SORT_WAVES);
+  sort_assign_kernel<W><<<blocks, SORT_THREADS, lds, stream>>>(idx, (const W*)w, M, k, E, nbits, (const int*)workspace,
+                                                               nvirtual, counts, offsets, token, (W*)wsorted, pos_of);
+  return sy_check_launch("sort_by_expert (assign)");
+}
+
+}  // namespace
+
+extern "C" SY_API size_t sy_sort_workspace_bytes(int N, int k, int E) {
+  const long M = (long)N * k;
+  if (N <= 0 || k <= 0 || E <= 0 || M <= SMALL_M) return 0;
+  return sizeof(int) * (size_t)large_blocks(M) * SORT_WAVES * E;
+}
+
+extern "C" SY_API int sy_sort_by_expert(const int32_t* idx, const void* w, int w_bytes, int N, int k, int E, int32_t* counts,
+                                 int32_t* offsets, int32_t* token, void* wsorted, int32_t* pos_of, void* workspace,
+                                 size_t workspace_bytes, void* stream) {
+  SY_REQUIRE(N >= 0 && k >= 1, "sort_by_expert: N = %d, k = %d", N, k);
+  SY_REQUIRE(E >= 1 && E <= MAX_E, "sort_by_expert: 1 <= E <= %d (got %d)", MAX_E, E);
+  SY_REQUIRE(w_bytes == 2 || w_bytes == 4, "sort_by_expert: weights of 2 or 4 bytes (got %d)", w_bytes);
+  SY_REQUIRE((long)N * k < (1l << 31) - SORT_THREADS * PIECE, "sort_by_expert: N*k too large");
+  SY_REQUIRE(counts && offsets, "sort_by_expert: null counts/offsets");
+  const int M = N * k;
+  SY_REQUIRE(M == 0 || (idx && w && token && wsorted && pos_of), "sort_by_expert: null pointer");
+  const size_t need = sy_sort_workspace_bytes(N, k, E);
+  SY_REQUIRE(need == 0 || (workspace && workspace_bytes >= need),
+             "sort_by_expert: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+  if (w_bytes == 2)
+    return launch_sort<uint16_t>(idx, w, M, k, E, counts, offsets, token, wsorted, pos_of, workspace,
+                                 (hipStream_t)stream);
+  return launch_sort<uint32_t>(idx, w, M, k, E, counts, offsets, token, wsorted, pos_of, workspace,
+                               (hipStream_t)stream);
+}

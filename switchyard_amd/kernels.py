@@ -1,0 +1,99 @@
+"""The MoE layer assembled from the gfx950 kernels: the same entry points, argument order and
+defaults as the reference's switchyard/kernels.py (:12-93), so `from switchyard_amd import
+kernels` stands in for `from switchyard import kernels`.
+
+Differences that follow from the hardware, none visible in the results:
+  - the native library is prebuilt C ABI + ctypes, not a JIT-built pybind module (`ext()`);
+  - "auto" never reads the per-expert counts back from the GPU (the reference waits on
+    `int(counts.max())`, kernels.py:86): it decides from the number of tokens, so a layer
+    enqueues its launches and returns;
+  - the grouped GEMM finds its row tiles on the device, so `tile_offsets` is kept only as a
+    helper with the reference's meaning and nothing here waits on `int(toff[-1])` (:61);
+  - `pick` never answers "cublas": the MFMA kernel covers that regime. The mode string
+    "cublas" is still accepted and runs the MFMA kernel.
+"""
+
+import torch
+import torch.nn.functional as F
+
+from . import _abi
+
+_EXT = None
+
+
+def ext():
+    global _EXT
+    if _EXT is None:
+        _EXT = _abi.Ext()
+    return _EXT
+
+
+def tile_offsets(counts, block=64):
+    tiles = (counts + block - 1) // block
+    off = torch.zeros(counts.numel() + 1, dtype=torch.int32, device=counts.device)
+    off[1:] = torch.cumsum(tiles, 0)
+    return off
+
+
+def route(h, router, top_k, norm_topk_prob):
+    """Returns (indices int32 [N, k], weights in h's dtype [N, k]); ties go to the lower expert id."""
+    return ext().route(F.linear(h, router).contiguous(), top_k, norm_topk_prob)
+
+
+# Measured on an MI355X with OLMoE's shapes (bench.py --sweep): the weight-stream kernel
+# handles 16 rows of an expert per pass and wins while experts have about that many rows;
+# beyond that the MFMA tile kernel does. There is no third regime on this hardware.
+GEMV_MAX_ROWS = 16
+GEMM_MAX_ROWS = 1 << 30
+
+
+def pick(max_rows):
+    if max_rows <= GEMV_MAX_ROWS:
+        return "gemv"
+    return "gemm"
+
+
+def _auto(n_tokens, n_choices, n_experts):
+    """Mode for "auto" without a device read. No expert can have more rows than there are
+    tokens, so up to GEMV_MAX_ROWS tokens the answer is certain; above that the mean rows
+    per expert stands in for the maximum (both kernels are correct for any routing)."""
+    if n_tokens <= GEMV_MAX_ROWS:
+        return "gemv"
+    return pick(-(-n_choices // n_experts))
+
+
+def ffn(x, a_rows, offsets, counts, wsorted, gate_up, down, rows, mode, host_counts=None):
+    """The experts over rows already sorted by expert: row i is x[a_rows[i]] (or x[i] when
+    a_rows is None); expert e owns rows offsets[e]:offsets[e+1]. Returns each row's expert
+    output scaled by its router weight, [rows, H]. `counts` and `host_counts` are accepted
+    for the reference's call shape; nothing here waits for the GPU."""
+    E = ext()
+    if rows == 0:
+        return torch.empty(0, down.shape[1], dtype=x.dtype, device=x.device)
+    if mode == "gemv":
+        act = E.grouped_gemv(x.contiguous(), a_rows, gate_up, offsets, rows, True, None)
+        return E.grouped_gemv(act, None, down, offsets, rows, False, wsorted)
+    if mode in ("gemm", "cublas"):
+        act = E.grouped_gemm(x.contiguous(), a_rows, gate_up, offsets, None, 0, rows, True, None)
+        return E.grouped_gemm(act, None, down, offsets, None, 0, rows, False, wsorted)
+    raise ValueError(f"unknown mode {mode!r}")
+
+
+def experts(h, idx, w, gate_up, down, mode="auto"):
+    """The experts of one MoE layer on this GPU, for routing (idx, w) computed already:
+    sort by expert, SwiGLU projection reading rows of h in place, down projection scaled by
+    the router weights, combine. idx int32 [N, k] in 0..E-1 local expert ids.
+    mode: "gemv" (streams weights; few rows per expert), "gemm" (MFMA tiles), or "auto"."""
+    E = ext()
+    N = h.shape[0]
+    idx = idx.contiguous()
+    counts, offsets, token, wsorted, pos_of = E.sort_by_expert(idx, w.contiguous(), gate_up.shape[0])
+    if mode == "auto":
+        mode = _auto(N, idx.numel(), gate_up.shape[0])
+    y = ffn(h, token, offsets, counts, wsorted, gate_up, down, idx.numel(), mode)
+    return E.combine(y, pos_of, idx, N)
+
+
+def moe_layer(h, router, gate_up, down, top_k, norm_topk_prob, mode="auto"):
+    idx, w = route(h, router, top_k, norm_topk_prob)
+    return experts(h, idx, w, gate_up, down, mode)

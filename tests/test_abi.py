@@ -1,0 +1,90 @@
+"""The C-ABI library loads without a GPU, exports every symbol the header declares, and
+rejects out-of-range arguments before touching the device. No compute is launched here."""
+
+import ctypes
+import os
+import re
+
+import pytest
+
+from switchyard_amd import _abi, kernels
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "switchyard_moe.h")
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return _abi.load_library()
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    return re.findall(r"^SY_API\s+[\w\s\*]+?\b(sy_\w+)\(", text, flags=re.M)
+
+
+def test_header_declares_the_expected_entry_points():
+    assert sorted(declared_symbols()) == sorted(["sy_version", "sy_last_error", "sy_route", "sy_sort_workspace_bytes",
+                                                  "sy_sort_by_expert", "sy_grouped_gemv", "sy_grouped_gemm",
+                                                  "sy_combine"])
+
+
+def test_library_exports_every_declared_symbol(lib):
+    raw = ctypes.CDLL(_abi.LIB_PATH)
+    for name in declared_symbols():
+        assert hasattr(raw, name), name
+        assert name in _abi.SIGNATURES, f"{name} has no ctypes signature"
+    assert lib.sy_version() >= 100
+
+
+def test_each_header_citation_names_a_reference_location():
+    text = open(HEADER).read()
+    for name in ("sy_route", "sy_sort_by_expert", "sy_grouped_gemv", "sy_grouped_gemm", "sy_combine"):
+        comment = text[:text.index(f"SY_API int {name}(")].rsplit("/*", 1)[1]
+        assert re.search(r"moe_kernels\.cu:\d+", comment), name
+
+
+def test_argument_errors_are_reported_without_a_device(lib):
+    assert lib.sy_route(None, 0, 5, 200, 8, 0, None, None, None) == 1
+    assert b"128 experts" in lib.sy_last_error()
+    assert lib.sy_route(None, 0, 5, 64, 9, 0, None, None, None) == 1
+    assert lib.sy_route(None, 7, 5, 64, 8, 0, None, None, None) == 1
+    assert lib.sy_grouped_gemm(None, None, None, None, 64, 5, 1024, 2040, 1, None, None, None) == 1
+    assert b"multiple of 32" in lib.sy_last_error()
+    assert lib.sy_grouped_gemv(None, None, None, None, 64, 5, 1024, 2044, 1, None, None, None) == 1
+    assert lib.sy_combine(None, None, None, 4, 8, 2044, None, None) == 1
+    assert lib.sy_combine(None, None, None, 4, 65, 2048, None, None) == 1
+    assert lib.sy_sort_by_expert(None, None, 3, 4, 8, 64, None, None, None, None, None, None, 0, None) == 1
+    assert lib.sy_sort_by_expert(None, None, 2, 4, 8, 513, None, None, None, None, None, None, 0, None) == 1
+
+
+def test_empty_inputs_are_no_ops(lib):
+    assert lib.sy_route(None, 0, 0, 64, 8, 0, None, None, None) == 0
+    assert lib.sy_grouped_gemv(None, None, None, None, 64, 0, 1024, 2048, 1, None, None, None) == 0
+    assert lib.sy_grouped_gemm(None, None, None, None, 64, 0, 1024, 2048, 1, None, None, None) == 0
+    assert lib.sy_combine(None, None, None, 0, 8, 2048, None, None) == 0
+
+
+def test_sort_workspace_grows_with_the_number_of_choices(lib):
+    assert lib.sy_sort_workspace_bytes(8, 8, 64) == 0
+    big = lib.sy_sort_workspace_bytes(4096, 8, 64)
+    assert big > 0 and lib.sy_sort_workspace_bytes(32768, 8, 64) > big
+
+
+def test_pick_and_tile_offsets_host_logic():
+    import torch
+
+    assert kernels.pick(1) == "gemv" and kernels.pick(kernels.GEMV_MAX_ROWS) == "gemv"
+    assert kernels.pick(kernels.GEMV_MAX_ROWS + 1) == "gemm" and kernels.pick(10 ** 6) == "gemm"
+    assert kernels._auto(8, 64, 64) == "gemv" and kernels._auto(4096, 32768, 64) == "gemm"
+    counts = torch.tensor([0, 1, 64, 65, 128, 0, 200])
+    assert kernels.tile_offsets(counts).tolist() == [0, 0, 1, 2, 4, 6, 6, 10]
+
+
+def test_host_wrappers_refuse_cpu_tensors():
+    import torch
+
+    with pytest.raises(RuntimeError, match="contiguous GPU tensor"):
+        kernels.ext().route(torch.zeros(4, 64, dtype=torch.float16), 8, False)
+    with pytest.raises(ValueError, match="unknown mode"):
+        kernels.ffn(torch.zeros(1, 8), None, None, None, None, None, torch.zeros(1, 8, 8), 1, "nope")
