@@ -66,9 +66,12 @@ SY_API int sy_sort_by_expert(const int32_t* idx, const void* w, int w_bytes, int
  * Nfull = 2*Nout when swiglu (gate rows first) else Nout; offsets int32 [E+1];
  * scale f16 [rows] or NULL; C f16 [rows,Nout].
  * swiglu: C = f16(f16(silu(f16(gate))) * f16(up)); scale: C = f16(f16(acc) * scale[r]).
- * Limits: K % 8 == 0, K <= 8192. rows == 0 is a no-op. */
+ * max_rows_hint: an upper bound on the rows of any one expert if the caller knows one (the
+ * number of tokens, when a token picks an expert at most once), else 0. It only sizes the
+ * kernel's row staging; results do not depend on it, and it need not hold.
+ * Limits: K % 8 == 0, K <= 4096. rows == 0 is a no-op. */
 SY_API int sy_grouped_gemv(const void* A, const int32_t* a_rows, const void* B, const int32_t* offsets, int E, int rows,
-                    int Nout, int K, int swiglu, const void* scale, void* C, void* stream);
+                           int max_rows_hint, int Nout, int K, int swiglu, const void* scale, void* C, void* stream);
 
 /* Replaces grouped_gemm() (moe_kernels.cu:264-298, kernel :167-261): the same function on
  * MFMA tiles for many rows per expert. The row tiles of every expert are derived from

@@ -27,7 +27,7 @@ SIGNATURES = {
     "sy_sort_by_expert": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p,
                                    _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_size_t, _c_void_p]),
     "sy_grouped_gemv": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int,
-                                 _c_void_p, _c_void_p, _c_void_p]),
+                                 _c_int, _c_void_p, _c_void_p, _c_void_p]),
     "sy_grouped_gemm": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int,
                                  _c_void_p, _c_void_p, _c_void_p]),
     "sy_combine": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p]),
@@ -108,7 +108,7 @@ class Ext:
                    ws.data_ptr() if need else None, need, _stream())
         return [counts, offsets, token, wsorted, pos_of]
 
-    def _grouped(self, fn, A, a_rows, B, offsets, rows, swiglu, scale):
+    def _grouped(self, fn, A, a_rows, B, offsets, rows, swiglu, scale, hint=None):
         _check(A, "A", torch.float16)
         _check(B, "B", torch.float16)
         _check(offsets, "offsets", torch.int32)
@@ -127,13 +127,16 @@ class Ext:
             raise RuntimeError("grouped: A has fewer rows than `rows`")
         Nout = Nfull // 2 if swiglu else Nfull
         C = torch.empty((rows, Nout), dtype=A.dtype, device=A.device)
+        extra = () if hint is None else (int(hint),)
         self._call(fn, A.data_ptr(), a_rows.data_ptr() if a_rows is not None else None, B.data_ptr(),
-                   offsets.data_ptr(), E, int(rows), Nout, K, int(bool(swiglu)),
+                   offsets.data_ptr(), E, int(rows), *extra, Nout, K, int(bool(swiglu)),
                    scale.data_ptr() if scale is not None else None, C.data_ptr(), _stream())
         return C
 
-    def grouped_gemv(self, A, a_rows, B, offsets, rows, swiglu, scale):
-        return self._grouped(self.lib.sy_grouped_gemv, A, a_rows, B, offsets, rows, swiglu, scale)
+    def grouped_gemv(self, A, a_rows, B, offsets, rows, swiglu, scale, max_rows=0):
+        """max_rows: an upper bound on the rows of one expert if known (0: unknown); a sizing
+        hint with no effect on the result."""
+        return self._grouped(self.lib.sy_grouped_gemv, A, a_rows, B, offsets, rows, swiglu, scale, hint=max_rows)
 
     def grouped_gemm(self, A, a_rows, B, offsets, tile_offsets, total_tiles, rows, swiglu, scale):
         """tile_offsets / total_tiles are accepted for the reference's call shape and unused:

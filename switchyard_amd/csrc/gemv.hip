@@ -1,21 +1,31 @@
 // grouped_gemv: the decode path. With a handful of rows per expert the layer is a stream over
-// the used experts' weights, so the kernel is built around that stream.
+// the used experts' weights, so the kernel is built around how HBM likes to be read.
 //
-// A workgroup of 4 wavefronts owns one expert and a run of 16-column groups of its weight
-// matrix. For a column group, lane (n = lane % 16, g = lane / 16) reads 16-byte pieces of
-// weight row col0 + n: the wavefronts split K between them in interleaved 32-wide steps, so
-// the workgroup as a whole reads 16 consecutive weight rows (one contiguous region of
-// 16*K*2 bytes) exactly once, every load 128 bits wide, and the pieces go from the load
-// straight into the MFMA operand registers (no LDS staging of weights).
+// Access pattern. A wavefront streams 4 consecutive weight rows (output columns) at a time,
+// sweeping along K. One 128-bit load instruction covers 4 rows x 256 contiguous bytes: lane
+// l = 4*b + i reads the 8 halves k = 8*b .. 8*b+7 (plus 128 per step) of row i. That footprint
+// (whole cache lines, four sequential streams) reads HBM about 25% faster than the 16 rows x
+// 64 bytes a 16x16 MFMA operand would ask for, and it is exactly the operand layout of
+// v_mfma_f32_4x4x4_16B_f16: 16 independent 4x4x4 products, block b of lanes 4b..4b+3. With
+// the weights as the 4 M rows and 4 of the expert's rows (tokens) as the N columns, block b
+// accumulates the partial dot products of its own slice of K; the loaded registers feed the
+// MFMA directly, the low and the high 4 halves in two instructions. At the end of K the 16
+// blocks are summed across lanes (a fixed tree, so results are deterministic) and lanes 0..3
+// hold 4 consecutive output columns of one row each. With SwiGLU a unit of work is the 4 gate
+// rows and then the 4 up rows of the same columns; the reduced gate values wait in registers.
 //
-// The expert's rows (up to 16 at a time) are the other MFMA operand: lane (n, g) holds row n
-// at the same K positions, loaded once per workgroup and kept in registers across all of its
-// column groups. v_mfma_f32_16x16x32_f16 then does the 16 rows x 16 columns of dot products
-// with fp32 accumulation: weights are the M operand and rows the N operand, so a lane ends
-// up with 4 consecutive output columns of one row. The 4 wavefronts' partial sums meet in
-// LDS (fixed order: deterministic) and wavefront 0 applies the epilogue and stores.
+// Balance. What a CU can pull from HBM is capped by the cache lines it may have in flight,
+// so the stream is only as fast as its slowest CU: every CU must be busy until the end. The
+// launch is therefore persistent, a fixed number of workgroups per CU, and the units of the
+// experts that received rows (found from `offsets` by every workgroup itself) are dealt to
+// the workgroups in equal contiguous shares. Experts without rows cost nothing.
 //
-// Experts without rows leave at once; an expert with more than 16 rows takes further passes.
+// Rows. The expert's rows (up to `row_cap` <= 16 per pass, in quads of 4) are staged in LDS,
+// padded so that the 128-bit operand reads are bank-conflict free, and shared by the
+// workgroup's 4 wavefronts, which split the units of the current expert between them and
+// otherwise run independently. Loads are issued one chunk (4 steps) ahead of the MFMAs that
+// consume them, through a buffer descriptor whose range check masks ragged edges without
+// branches. An expert with more rows than `row_cap` takes further passes over its weights.
 //
 // Replaces grouped_gemv_kernel / grouped_gemv of the reference
 // (switchyard/csrc/moe_kernels.cu:301-415); epilogue rounding points as :373-378.
@@ -23,15 +33,23 @@
 
 namespace {
 
-constexpr int GEMV_WAVES = 4;
+constexpr int GEMV_WAVES = 4;   // wavefronts per workgroup (they share the staged rows)
 constexpr int GEMV_THREADS = GEMV_WAVES * WAVE;
-constexpr int GEMV_ROWS = 16;   // rows per pass (MFMA N)
-constexpr int GEMV_COLS = 16;   // columns per group (MFMA M)
-constexpr int GEMV_MAX_KS = 16; // 32-wide K steps a wavefront keeps in registers
+constexpr int UNIT_COLS = 4;    // output columns per unit (MFMA M)
+constexpr int QUAD = 4;         // rows of the expert per MFMA (MFMA N)
+constexpr int MAX_QUADS = 4;    // up to 16 rows per pass
+constexpr int STEP_K = 128;     // K covered by one load instruction (16 blocks x 8 halves)
+constexpr int CH = 4;           // load steps per chunk
+constexpr int ROW_PAD = 32;     // halves of padding per staged row (64 bytes)
+constexpr int MAX_E = 1024;     // experts whose ids fit the LDS list
+constexpr int BLOCKS_PER_CU = 2;
 
-__device__ __forceinline__ half8_t load_stream(const half_t* p) {
-  return __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(p));
+// 128-bit streaming load through a buffer descriptor: lane offset in bytes (out of range
+// reads return 0), wave-uniform offset in an SGPR.
+__device__ __forceinline__ half8_t load_stream(__amdgpu_buffer_rsrc_t rsrc, unsigned lane_off, unsigned uniform_off) {
+  return __builtin_bit_cast(half8_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_off, uniform_off, /*nt*/ 2));
 }
+constexpr unsigned OUT_OF_RANGE = 0x80000000u;
 
 __device__ __forceinline__ half_t swiglu_f16(float gate, float up) {
   // the rounding points of the fp16 torch graph: gate and up to f16, silu in fp32 to f16, product to f16
@@ -40,133 +58,274 @@ __device__ __forceinline__ half_t swiglu_f16(float gate, float up) {
   return (half_t)(s * u);
 }
 
-template <int KS, bool SWIGLU, bool SCALE>
-__global__ void __launch_bounds__(GEMV_THREADS)
-gemv_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const half_t* __restrict__ B,
-            const int* __restrict__ offsets, int Nout, int K, const half_t* __restrict__ scale,
-            half_t* __restrict__ C, int groups_per_block) {
-  const int e = blockIdx.y;
-  const int start = offsets[e], end = offsets[e + 1];
-  if (start >= end) return;
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, n = lane & 15, g = lane >> 4;
-  const int Nfull = SWIGLU ? 2 * Nout : Nout;
-  const half_t* Be = B + (size_t)e * Nfull * K;
-  constexpr int NACC = SWIGLU ? 2 : 1;
-  __shared__ float4_t part[2][GEMV_WAVES][NACC][WAVE];
+__device__ __forceinline__ half4_t lo4(half8_t v) { return __builtin_shufflevector(v, v, 0, 1, 2, 3); }
+__device__ __forceinline__ half4_t hi4(half8_t v) { return __builtin_shufflevector(v, v, 4, 5, 6, 7); }
 
-  const int ngroups = (Nout + GEMV_COLS - 1) / GEMV_COLS;
-  const int cg0 = blockIdx.x * groups_per_block, cg1 = min(cg0 + groups_per_block, ngroups);
-  constexpr int SUPER = GEMV_WAVES * KS * 32;  // K covered by one register-resident set of steps
-  const int nsuper = (K + SUPER - 1) / SUPER;
+// Sum over the 16 blocks (lanes with equal lane % 4); lanes 0..3 end with the total.
+__device__ __forceinline__ float sum_blocks(float v) {
+  v += dpp_row_ror<4>(v);
+  v += dpp_row_ror<8>(v);   // every lane: the sum over its row of 16 lanes (4 blocks)
+  v += __shfl_down(v, 32, WAVE);
+  v += __shfl_down(v, 16, WAVE);
+  return v;
+}
+
+struct Chunk {
+  half8_t w[CH];
+};
+
+struct Pass {
+  const half_t* xs;             // staged rows
+  __amdgpu_buffer_rsrc_t rsrc;  // the expert's weight matrix
+  const half_t* scale;
+  half_t* C;
+  int Nout, K, RS, r0, nr, unit0, nunits, nchunks;
+};
+
+// One wavefront streams units [unit0, unit0 + nunits) of one expert against NQ staged quads.
+// EXACT: K is a multiple of a chunk (512) and Nout of a unit (4), so nothing needs masking.
+template <bool SWIGLU, bool SCALE, bool EXACT, int NQ>
+__device__ __forceinline__ void run_pass(const Pass& p) {
+  const int lane = threadIdx.x & 63, blk = lane >> 2, sub = lane & 3;
+  const int klane = blk * 8;
+  constexpr int PARTS = SWIGLU ? 2 : 1;  // a unit is streamed as its gate rows, then its up rows
   const half8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-  int flip = 0;
 
-  for (int r0 = start; r0 < end; r0 += GEMV_ROWS) {
-    const int nr = min(GEMV_ROWS, end - r0);
-    const half_t* xrow = nullptr;
-    if (n < nr) xrow = A + (size_t)(a_rows ? a_rows[r0 + n] : r0 + n) * K;
-    half8_t xf[KS];
-    auto load_rows = [&](int sc) {
+  // ---- issue side: part `ipt` of unit `iun`, chunk `ich` is the next to load
+  int iun = 0, ipt = 0, ich = 0;
+  auto issue = [&](Chunk& c) {
+    const int col = (p.unit0 + iun) * UNIT_COLS + sub;
+    const int wr = ipt ? p.Nout + col : col;
+    unsigned lane_off = ((unsigned)wr * (unsigned)p.K + (unsigned)klane) * 2u;
+    if (!EXACT && col >= p.Nout) lane_off = OUT_OF_RANGE;
 #pragma unroll
-      for (int s = 0; s < KS; ++s) {
-        const int kk = sc * SUPER + (s * GEMV_WAVES + wave) * 32 + g * 8;
-        xf[s] = (xrow && kk < K) ? *reinterpret_cast<const half8_t*>(xrow + kk) : zero8;
+    for (int s = 0; s < CH; ++s) {
+      const int kk = (ich * CH + s) * STEP_K;
+      unsigned off = lane_off;
+      if (!EXACT && kk + klane >= p.K) off = OUT_OF_RANGE;
+      c.w[s] = load_stream(p.rsrc, off, (unsigned)kk * 2u);
+    }
+    if (++ich == p.nchunks) {
+      ich = 0;
+      if (++ipt == PARTS) {
+        ipt = 0;
+        ++iun;
       }
-    };
-    if (nsuper == 1) load_rows(0);
+    }
+  };
 
-    for (int cg = cg0; cg < cg1; ++cg) {
-      const int col = cg * GEMV_COLS + n;
-      const bool colok = col < Nout;
-      const half_t* wrow = Be + (size_t)col * K;
-      const half_t* urow = Be + (size_t)(Nout + col) * K;
-      float4_t accg = {0.f, 0.f, 0.f, 0.f}, accu = {0.f, 0.f, 0.f, 0.f};
-      for (int sc = 0; sc < nsuper; ++sc) {
-        if (nsuper > 1) load_rows(sc);
-        half8_t wg[KS], wu[KS];
+  // ---- compute side
+  int cun = 0, cpt = 0, cch = 0;
+  float4_t acc[NQ], gate[NQ];
 #pragma unroll
-        for (int s = 0; s < KS; ++s) {
-          const int kk = sc * SUPER + (s * GEMV_WAVES + wave) * 32 + g * 8;
-          const bool ok = colok && kk < K;
-          wg[s] = ok ? load_stream(wrow + kk) : zero8;
-          if (SWIGLU) wu[s] = ok ? load_stream(urow + kk) : zero8;
-        }
+  for (int q = 0; q < NQ; ++q) acc[q] = gate[q] = float4_t{0.f, 0.f, 0.f, 0.f};
+  const half_t* xlane = p.xs + sub * p.RS + klane;  // row `sub` of quad 0 at this lane's K offset
+
+  auto compute = [&](const Chunk& c) {
 #pragma unroll
-        for (int s = 0; s < KS; ++s) {
-          accg = __builtin_amdgcn_mfma_f32_16x16x32_f16(wg[s], xf[s], accg, 0, 0, 0);
-          if (SWIGLU) accu = __builtin_amdgcn_mfma_f32_16x16x32_f16(wu[s], xf[s], accu, 0, 0, 0);
-        }
+    for (int s = 0; s < CH; ++s) {
+      const int kk = (cch * CH + s) * STEP_K;
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) {
+        half8_t x = *reinterpret_cast<const half8_t*>(xlane + q * QUAD * p.RS + kk);
+        if (!EXACT && kk + klane >= p.K) x = zero8;  // the weights are 0 there; keep stale LDS out
+        acc[q] = __builtin_amdgcn_mfma_f32_4x4x4f16(lo4(c.w[s]), lo4(x), acc[q], 0, 0, 0);
+        acc[q] = __builtin_amdgcn_mfma_f32_4x4x4f16(hi4(c.w[s]), hi4(x), acc[q], 0, 0, 0);
       }
-      part[flip][wave][0][lane] = accg;
-      if (SWIGLU) part[flip][wave][NACC - 1][lane] = accu;
-      __syncthreads();
-      if (wave == 0 && n < nr) {
-        float4_t sg = part[flip][0][0][lane], su = {0.f, 0.f, 0.f, 0.f};
-        if (SWIGLU) su = part[flip][0][NACC - 1][lane];
+    }
+    if (++cch < p.nchunks) return;
+    cch = 0;
+    // part done: sum the 16 K-slices; lane j < 4 then holds columns c0..c0+3 of row 4q + j
+    const bool is_gate = SWIGLU && cpt == 0;
+    const int c0 = (p.unit0 + cun) * UNIT_COLS;
 #pragma unroll
-        for (int wv = 1; wv < GEMV_WAVES; ++wv) {
-          sg += part[flip][wv][0][lane];
-          if (SWIGLU) su += part[flip][wv][NACC - 1][lane];
-        }
-        const int row = r0 + n, c0 = cg * GEMV_COLS + 4 * g;
-        const float sc_row = SCALE ? (float)scale[row] : 1.f;
+    for (int q = 0; q < NQ; ++q) {
+      float4_t v;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = sum_blocks(acc[q][i]);
+      acc[q] = float4_t{0.f, 0.f, 0.f, 0.f};
+      if (is_gate) {
+        gate[q] = v;
+        continue;
+      }
+      const int r = q * QUAD + lane;
+      if (lane < QUAD && r < p.nr) {
+        const float row_scale = SCALE ? (float)p.scale[p.r0 + r] : 1.f;
         half4_t o;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          if (SWIGLU) o[i] = swiglu_f16(sg[i], su[i]);
-          else if (SCALE) o[i] = (half_t)((float)(half_t)sg[i] * sc_row);
-          else o[i] = (half_t)sg[i];
+          if (SWIGLU) o[i] = swiglu_f16(gate[q][i], v[i]);
+          else if (SCALE) o[i] = (half_t)((float)(half_t)v[i] * row_scale);
+          else o[i] = (half_t)v[i];
         }
-        half_t* dst = C + (size_t)row * Nout + c0;
-        if (c0 + 3 < Nout && (Nout & 3) == 0) {
+        half_t* dst = p.C + (size_t)(p.r0 + r) * p.Nout + c0;
+        if (EXACT || (c0 + 3 < p.Nout && (p.Nout & 3) == 0)) {
           *reinterpret_cast<half4_t*>(dst) = o;
         } else {
 #pragma unroll
           for (int i = 0; i < 4; ++i)
-            if (c0 + i < Nout) dst[i] = o[i];
+            if (c0 + i < p.Nout) dst[i] = o[i];
         }
       }
-      flip ^= 1;
     }
+    if (++cpt == PARTS) {
+      cpt = 0;
+      ++cun;
+    }
+  };
+
+  // chunk q+1 is in flight while chunk q is multiplied
+  const int total = p.nunits * PARTS * p.nchunks;
+  if (total <= 0) return;
+  Chunk c0, c1;
+  issue(c0);
+  int q = 0;
+  for (; q + 3 <= total; q += 2) {
+    issue(c1);
+    compute(c0);
+    issue(c0);
+    compute(c1);
+  }
+  if (total - q == 2) {
+    issue(c1);
+    compute(c0);
+    compute(c1);
+  } else {
+    compute(c0);
   }
 }
 
-template <int KS>
-int launch_gemv(const void* A, const int32_t* a_rows, const void* B, const int32_t* offsets, int E, int Nout, int K,
-                int swiglu, const void* scale, void* C, hipStream_t stream) {
-  const int ngroups = (Nout + GEMV_COLS - 1) / GEMV_COLS;
-  // about 128 KB of weights per workgroup
-  const long group_bytes = (long)GEMV_COLS * K * 2 * (swiglu ? 2 : 1);
-  int gpb = (int)((128 * 1024 + group_bytes - 1) / group_bytes);
-  gpb = gpb < 1 ? 1 : (gpb > ngroups ? ngroups : gpb);
-  const dim3 grid((ngroups + gpb - 1) / gpb, E);
+template <bool SWIGLU, bool SCALE, bool EXACT>
+__global__ void __launch_bounds__(GEMV_THREADS)
+gemv_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const half_t* __restrict__ B,
+            const int* __restrict__ offsets, int E, int Nout, int K, const half_t* __restrict__ scale,
+            half_t* __restrict__ C, int row_cap) {
+  extern __shared__ __attribute__((aligned(16))) half_t xs[];  // [row_cap][K + ROW_PAD], then the used experts
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int RS = K + ROW_PAD;
+  int* used = reinterpret_cast<int*>(xs + (size_t)row_cap * RS);  // [E] ids of experts with rows, [E] = how many
+  const half8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  // ---- the experts that received rows, in order (one wavefront, 64 experts per step)
+  if (wave == 0) {
+    int n = 0;
+    for (int e0 = 0; e0 < E; e0 += WAVE) {
+      const int e = e0 + lane;
+      const bool has = e < E && offsets[e + 1] > offsets[e];
+      const uint64_t m = __ballot(has);
+      if (has) used[n + __popcll(m & lanemask_lt())] = e;
+      n += __popcll(m);
+    }
+    if (lane == 0) used[E] = n;
+  }
+  __syncthreads();
+  const int nused = used[E];
+  const int units_per_expert = (Nout + UNIT_COLS - 1) / UNIT_COLS;
+
+  // ---- this workgroup's equal share of all units, a contiguous range [lo, hi)
+  const long total_units = (long)nused * units_per_expert;
+  const int lo = (int)(total_units * blockIdx.x / gridDim.x), hi = (int)(total_units * (blockIdx.x + 1) / gridDim.x);
+
+  Pass p;
+  p.xs = xs;
+  p.Nout = Nout;
+  p.K = K;
+  p.RS = RS;
+  p.scale = scale;
+  p.C = C;
+  p.nchunks = ((K + STEP_K - 1) / STEP_K + CH - 1) / CH;
+  const int Nfull = SWIGLU ? 2 * Nout : Nout;
+  bool staged = false;
+
+  for (int at = lo; at < hi;) {
+    // the part of the range that falls into one expert
+    const int u = at / units_per_expert, first = at - u * units_per_expert;
+    const int count = min(hi - at, units_per_expert - first);
+    const int e = used[u];
+    const int start = offsets[e], end = offsets[e + 1];
+    p.rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(B + (size_t)e * Nfull * K), 0,
+                                               (int)((size_t)Nfull * K * 2), 0x00020000);
+    // wavefront w takes a contiguous quarter of the units
+    p.unit0 = first + (int)((long)count * wave / GEMV_WAVES);
+    p.nunits = first + (int)((long)count * (wave + 1) / GEMV_WAVES) - p.unit0;
+
+    for (int r0 = start; r0 < end; r0 += row_cap) {
+      const int nr = min(row_cap, end - r0);
+      const int nq = (nr + QUAD - 1) / QUAD;
+      // ---- stage the pass's rows: wavefront w copies rows w, w+4, ...; missing rows of the last quad are zero
+      if (staged) __syncthreads();
+      for (int r = wave; r < nq * QUAD; r += GEMV_WAVES) {
+        const half_t* src = r < nr ? A + (size_t)(a_rows ? a_rows[r0 + r] : r0 + r) * K : nullptr;
+        for (int kk = lane * 8; kk < K; kk += WAVE * 8)
+          *reinterpret_cast<half8_t*>(xs + r * RS + kk) = src ? *reinterpret_cast<const half8_t*>(src + kk) : zero8;
+      }
+      __syncthreads();
+      staged = true;
+      p.r0 = r0;
+      p.nr = nr;
+      switch (nq) {
+        case 1: run_pass<SWIGLU, SCALE, EXACT, 1>(p); break;
+        case 2: run_pass<SWIGLU, SCALE, EXACT, 2>(p); break;
+        case 3: run_pass<SWIGLU, SCALE, EXACT, 3>(p); break;
+        default: run_pass<SWIGLU, SCALE, EXACT, 4>(p); break;
+      }
+    }
+    at += count;
+  }
+}
+
+// Compute units of the current device (cached per device id; read-only after the first call).
+int compute_units() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
+int launch_gemv(const void* A, const int32_t* a_rows, const void* B, const int32_t* offsets, int E, int rows,
+                int max_rows_hint, int Nout, int K, int swiglu, const void* scale, void* C, hipStream_t stream) {
+  // rows staged per pass: no expert has more rows than there are rows in all; a caller that
+  // knows a tighter bound (the number of tokens) saves LDS and gains occupancy
+  const int bound = max_rows_hint > 0 && max_rows_hint < rows ? max_rows_hint : rows;
+  int row_cap = (bound + QUAD - 1) / QUAD * QUAD;
+  row_cap = row_cap > MAX_QUADS * QUAD ? MAX_QUADS * QUAD : row_cap;
+  const size_t lds = (size_t)row_cap * (K + ROW_PAD) * sizeof(half_t) + (size_t)(E + 1) * sizeof(int);
+  // persistent: a fixed number of workgroups per CU, but no more than there are units
+  const long max_units = (long)(E < rows ? E : rows) * ((Nout + UNIT_COLS - 1) / UNIT_COLS);
+  long grid = (long)compute_units() * BLOCKS_PER_CU;
+  grid = grid > max_units ? max_units : grid;
   const half_t* a = (const half_t*)A;
   const half_t* b = (const half_t*)B;
   const half_t* s = (const half_t*)scale;
   half_t* c = (half_t*)C;
-  if (swiglu)
-    gemv_kernel<KS, true, false><<<grid, GEMV_THREADS, 0, stream>>>(a, a_rows, b, offsets, Nout, K, nullptr, c, gpb);
-  else if (s)
-    gemv_kernel<KS, false, true><<<grid, GEMV_THREADS, 0, stream>>>(a, a_rows, b, offsets, Nout, K, s, c, gpb);
-  else
-    gemv_kernel<KS, false, false><<<grid, GEMV_THREADS, 0, stream>>>(a, a_rows, b, offsets, Nout, K, nullptr, c, gpb);
+  const bool exact = K % (CH * STEP_K) == 0 && Nout % UNIT_COLS == 0;
+  void (*kern)(const half_t*, const int*, const half_t*, const int*, int, int, int, const half_t*, half_t*, int);
+  if (swiglu) kern = exact ? gemv_kernel<true, false, true> : gemv_kernel<true, false, false>;
+  else if (s) kern = exact ? gemv_kernel<false, true, true> : gemv_kernel<false, true, false>;
+  else kern = exact ? gemv_kernel<false, false, true> : gemv_kernel<false, false, false>;
+  hipError_t attr = hipSuccess;
+  if (lds > 48 * 1024) attr = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (attr != hipSuccess) return sy_fail(SY_ERR_LAUNCH, "grouped_gemv: cannot reserve %zu bytes of LDS", lds);
+  kern<<<(unsigned)grid, GEMV_THREADS, lds, stream>>>(a, a_rows, b, offsets, E, Nout, K, swiglu ? nullptr : s, c, row_cap);
   return sy_check_launch("grouped_gemv");
 }
 
 }  // namespace
 
-extern "C" SY_API int sy_grouped_gemv(const void* A, const int32_t* a_rows, const void* B, const int32_t* offsets, int E,
-                               int rows, int Nout, int K, int swiglu, const void* scale, void* C, void* stream) {
-  SY_REQUIRE(rows >= 0 && E >= 1 && E <= 65535 && Nout >= 1, "grouped_gemv: rows = %d, E = %d, Nout = %d", rows, E, Nout);
-  SY_REQUIRE(K >= 8 && K % 8 == 0 && K <= 8192, "grouped_gemv: K must be a multiple of 8 up to 8192 (got %d)", K);
+extern "C" SY_API int sy_grouped_gemv(const void* A, const int32_t* a_rows, const void* B, const int32_t* offsets,
+                                      int E, int rows, int max_rows_hint, int Nout, int K, int swiglu,
+                                      const void* scale, void* C, void* stream) {
+  SY_REQUIRE(rows >= 0 && E >= 1 && E <= MAX_E && Nout >= 1, "grouped_gemv: rows = %d, E = %d (at most %d), Nout = %d",
+             rows, E, MAX_E, Nout);
+  SY_REQUIRE(K >= 8 && K % 8 == 0 && K <= 4096, "grouped_gemv: K must be a multiple of 8 up to 4096 (got %d)", K);
+  SY_REQUIRE((long)Nout * K * (swiglu ? 4 : 2) < (1l << 31), "grouped_gemv: an expert's matrix must stay under 2 GiB");
   SY_REQUIRE(!(swiglu && scale), "grouped_gemv: swiglu and scale are not combined");
   if (rows == 0) return SY_OK;
   SY_REQUIRE(A && B && offsets && C, "grouped_gemv: null pointer");
-  const int per_wave = ((K + 31) / 32 + GEMV_WAVES - 1) / GEMV_WAVES;
-  hipStream_t st = (hipStream_t)stream;
-  if (per_wave <= 1) return launch_gemv<1>(A, a_rows, B, offsets, E, Nout, K, swiglu, scale, C, st);
-  if (per_wave <= 2) return launch_gemv<2>(A, a_rows, B, offsets, E, Nout, K, swiglu, scale, C, st);
-  if (per_wave <= 4) return launch_gemv<4>(A, a_rows, B, offsets, E, Nout, K, swiglu, scale, C, st);
-  if (per_wave <= 8) return launch_gemv<8>(A, a_rows, B, offsets, E, Nout, K, swiglu, scale, C, st);
-  return launch_gemv<GEMV_MAX_KS>(A, a_rows, B, offsets, E, Nout, K, swiglu, scale, C, st);
+  return launch_gemv(A, a_rows, B, offsets, E, rows, max_rows_hint, Nout, K, swiglu, scale, C, (hipStream_t)stream);
 }

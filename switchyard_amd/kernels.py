@@ -71,8 +71,10 @@ def ffn(x, a_rows, offsets, counts, wsorted, gate_up, down, rows, mode, host_cou
     if rows == 0:
         return torch.empty(0, down.shape[1], dtype=x.dtype, device=x.device)
     if mode == "gemv":
-        act = E.grouped_gemv(x.contiguous(), a_rows, gate_up, offsets, rows, True, None)
-        return E.grouped_gemv(act, None, down, offsets, rows, False, wsorted)
+        # a token picks an expert at most once, so no expert has more rows than x has tokens
+        bound = x.shape[0] if a_rows is not None else 0
+        act = E.grouped_gemv(x.contiguous(), a_rows, gate_up, offsets, rows, True, None, bound)
+        return E.grouped_gemv(act, None, down, offsets, rows, False, wsorted, bound)
     if mode in ("gemm", "cublas"):
         act = E.grouped_gemm(x.contiguous(), a_rows, gate_up, offsets, None, 0, rows, True, None)
         return E.grouped_gemm(act, None, down, offsets, None, 0, rows, False, wsorted)

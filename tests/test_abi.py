@@ -51,7 +51,7 @@ def test_argument_errors_are_reported_without_a_device(lib):
     assert lib.sy_route(None, 7, 5, 64, 8, 0, None, None, None) == 1
     assert lib.sy_grouped_gemm(None, None, None, None, 64, 5, 1024, 2040, 1, None, None, None) == 1
     assert b"multiple of 32" in lib.sy_last_error()
-    assert lib.sy_grouped_gemv(None, None, None, None, 64, 5, 1024, 2044, 1, None, None, None) == 1
+    assert lib.sy_grouped_gemv(None, None, None, None, 64, 5, 0, 1024, 2044, 1, None, None, None) == 1
     assert lib.sy_combine(None, None, None, 4, 8, 2044, None, None) == 1
     assert lib.sy_combine(None, None, None, 4, 65, 2048, None, None) == 1
     assert lib.sy_sort_by_expert(None, None, 3, 4, 8, 64, None, None, None, None, None, None, 0, None) == 1
@@ -60,7 +60,7 @@ def test_argument_errors_are_reported_without_a_device(lib):
 
 def test_empty_inputs_are_no_ops(lib):
     assert lib.sy_route(None, 0, 0, 64, 8, 0, None, None, None) == 0
-    assert lib.sy_grouped_gemv(None, None, None, None, 64, 0, 1024, 2048, 1, None, None, None) == 0
+    assert lib.sy_grouped_gemv(None, None, None, None, 64, 0, 0, 1024, 2048, 1, None, None, None) == 0
     assert lib.sy_grouped_gemm(None, None, None, None, 64, 0, 1024, 2048, 1, None, None, None) == 0
     assert lib.sy_combine(None, None, None, 0, 8, 2048, None, None) == 0
 
