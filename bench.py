@@ -54,7 +54,8 @@ def hidden(N, seed=0):
 
 
 def event_times(fn, reps):
-    """Per-call GPU time in ms, one event pair per call on the current stream."""
+    """Per-call GPU time in ms, one event pair per call on the current stream (the GPU idles
+    between calls, so launch latency is included: the reference's bench/kernels.py method)."""
     out = []
     for _ in range(reps):
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -64,6 +65,19 @@ def event_times(fn, reps):
         b.synchronize()
         out.append(a.elapsed_time(b))
     return out
+
+
+def stream_times(fn, reps):
+    """Per-launch GPU time in ms for back-to-back launches: events are recorded in the stream
+    between launches and read after one synchronize, so the queue never drains and each
+    interval is one launch (kernel time plus the dispatch gap)."""
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(reps + 1)]
+    ev[0].record()
+    for i in range(reps):
+        fn()
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    return [ev[i].elapsed_time(ev[i + 1]) for i in range(reps)]
 
 
 def cpu_loop_baseline(h, router, gu, dn, used, reps=5):
@@ -140,13 +154,13 @@ def run_default(args):
         g_, off_, tok_ = rot[calls[0] % len(rot)]
         calls[0] += 1
         if use_gemv:
-            return kernels.ext().grouped_gemv(h, tok_, g_, off_, M, True, None)
+            return kernels.ext().grouped_gemv(h, tok_, g_, off_, M, True, None, N)
         return kernels.ext().grouped_gemm(h, tok_, g_, off_, None, 0, M, True, None)
 
     for _ in range(max(3, args.warmup)):
         gate_up()
     calls[0] = 0
-    kt = event_times(gate_up, max(args.steps, 20))
+    kt = stream_times(gate_up, max(args.steps, 20))
     k_ms = sum(kt) / len(kt)
     used_k = sum(used[j % len(layers)] for j in range(len(kt))) / len(kt)
     if use_gemv or M // E < 300:

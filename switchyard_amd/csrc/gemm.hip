@@ -1,18 +1,19 @@
 // grouped_gemm: the prefill path. Every expert's slice of the sorted rows goes through that
 // expert's weights on fp16 MFMA tiles, all experts in one launch.
 //
-// Tile: 128 rows x 256 weight rows, K in slices of 32, 4 wavefronts (2 x 2), each computing
+// Tile: 128 rows x 256 weight rows, K in slices of 64, 4 wavefronts (2 x 2), each computing
 // 64 rows x 128 weight rows as 2 x 4 v_mfma_f32_32x32x16_f16 blocks with fp32 accumulators.
 // With SwiGLU the 256 weight rows are 128 gate rows and the 128 up rows of the same output
 // columns, and a wavefront holds gate and up of the same 64 columns, so the activation is
 // applied in registers. Weights are the MFMA M operand and rows the N operand: a lane ends
 // up with runs of 4 consecutive output columns of one row and stores them as 8 bytes.
 //
-// Rows are gathered from the unsorted input inside the kernel (a_rows). K-slices are
-// double-buffered in LDS: while the MFMAs consume slice i from one buffer, the global loads
-// of slice i+1 are in flight into registers and are written to the other buffer afterwards,
-// one barrier per slice. LDS rows are padded to 80 bytes so that the 128-bit operand reads
-// of 16 consecutive lanes fall in distinct banks.
+// Rows are gathered from the unsorted input inside the kernel (a_rows). A K-slice is 64 wide
+// so that every row contributes a whole 128-byte cache line per slice. While the MFMAs
+// consume slice i from LDS, the global loads of slice i+1 are in flight into registers; they
+// are written to LDS between two barriers, and the second workgroup resident on the CU
+// computes meanwhile. LDS rows are padded to 144 bytes so that the 128-bit operand reads of
+// 16 consecutive lanes fall in distinct banks.
 //
 // The row tiles of all experts are laid end to end. The map from a tile to (expert, first
 // row) is rebuilt by every workgroup from `offsets` with one wavefront scan, so the host
@@ -29,8 +30,8 @@ namespace {
 
 constexpr int BM = 128;          // rows per tile
 constexpr int BW = 256;          // weight rows per tile
-constexpr int BK = 32;           // K per slice
-constexpr int LDS_LD = BK + 8;   // halves per LDS row (80 bytes)
+constexpr int BK = 64;           // K per slice
+constexpr int LDS_LD = BK + 8;   // halves per LDS row (144 bytes)
 constexpr int GEMM_THREADS = 256;
 constexpr int XCDS = 8;
 
@@ -45,7 +46,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 2)
 gemm_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const half_t* __restrict__ B,
             const int* __restrict__ offsets, int E, int Nout, int K, const half_t* __restrict__ scale,
             half_t* __restrict__ C, int ncol_tiles, int per_xcd) {
-  __shared__ __attribute__((aligned(16))) half_t lds[2][(BM + BW) * LDS_LD];
+  __shared__ __attribute__((aligned(16))) half_t lds[(BM + BW) * LDS_LD];
   __shared__ int s_tile[3];
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -87,18 +88,19 @@ gemm_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const 
   const int Nfull = SWIGLU ? 2 * Nout : Nout;
   const half_t* Be = B + (size_t)e * Nfull * K;
 
-  // ---- loader: thread t moves 16-byte chunk (t & 3) of rows (t >> 2) + 64*q
-  const int lrow = tid >> 2, lch = (tid & 3) * 8;
-  const half_t* pa[2];
-  const half_t* pb[4];
+  // ---- loader: thread t moves 16-byte chunk (t & 7) of rows (t >> 3) + 32*q
+  const int lrow = tid >> 3, lch = (tid & 7) * 8;
+  constexpr int NA = BM / 32, NB = BW / 32;
+  const half_t* pa[NA];
+  const half_t* pb[NB];
 #pragma unroll
-  for (int q = 0; q < 2; ++q) {
-    const int r = lrow + 64 * q;
+  for (int q = 0; q < NA; ++q) {
+    const int r = lrow + 32 * q;
     pa[q] = r < nrows ? A + (size_t)(a_rows ? a_rows[row0 + r] : row0 + r) * K + lch : nullptr;
   }
 #pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    const int br = lrow + 64 * q;
+  for (int q = 0; q < NB; ++q) {
+    const int br = lrow + 32 * q;
     int wr, col;
     if (SWIGLU) {
       col = n0 + (br & (COLS - 1));
@@ -110,20 +112,21 @@ gemm_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const 
     pb[q] = col < Nout ? Be + (size_t)wr * K + lch : nullptr;
   }
   const half8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-  half8_t ra[2], rb[4];
+  half8_t ra[NA], rb[NB];
   auto fetch = [&](int k0) {
+    const bool kok = k0 + lch < K;  // K may end in the middle of the last slice
 #pragma unroll
-    for (int q = 0; q < 2; ++q) ra[q] = pa[q] ? *reinterpret_cast<const half8_t*>(pa[q] + k0) : zero8;
+    for (int q = 0; q < NA; ++q) ra[q] = (pa[q] && kok) ? *reinterpret_cast<const half8_t*>(pa[q] + k0) : zero8;
 #pragma unroll
-    for (int q = 0; q < 4; ++q) rb[q] = pb[q] ? *reinterpret_cast<const half8_t*>(pb[q] + k0) : zero8;
+    for (int q = 0; q < NB; ++q) rb[q] = (pb[q] && kok) ? *reinterpret_cast<const half8_t*>(pb[q] + k0) : zero8;
   };
-  auto stash = [&](int buf) {
-    half_t* as = lds[buf];
+  auto stash = [&]() {
+    half_t* as = lds;
     half_t* bs = as + BM * LDS_LD;
 #pragma unroll
-    for (int q = 0; q < 2; ++q) *reinterpret_cast<half8_t*>(as + (lrow + 64 * q) * LDS_LD + lch) = ra[q];
+    for (int q = 0; q < NA; ++q) *reinterpret_cast<half8_t*>(as + (lrow + 32 * q) * LDS_LD + lch) = ra[q];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) *reinterpret_cast<half8_t*>(bs + (lrow + 64 * q) * LDS_LD + lch) = rb[q];
+    for (int q = 0; q < NB; ++q) *reinterpret_cast<half8_t*>(bs + (lrow + 32 * q) * LDS_LD + lch) = rb[q];
   };
 
   // ---- wavefront tile
@@ -142,14 +145,14 @@ gemm_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const 
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   fetch(0);
-  stash(0);
-  __syncthreads();
-  const int nk = K / BK;
+  const int nk = (K + BK - 1) / BK;
+  const half_t* as = lds + (wm * 64 + l32) * LDS_LD + lk;
+  const half_t* bs = lds + (BM + l32) * LDS_LD + lk;
   for (int kt = 0; kt < nk; ++kt) {
-    const int buf = kt & 1;
+    if (kt) __syncthreads();  // every wavefront is done reading the previous slice
+    stash();
+    __syncthreads();
     if (kt + 1 < nk) fetch((kt + 1) * BK);
-    const half_t* as = lds[buf] + (wm * 64 + l32) * LDS_LD + lk;
-    const half_t* bs = lds[buf] + (BM + l32) * LDS_LD + lk;
 #pragma unroll
     for (int kk = 0; kk < BK; kk += 16) {
       half8_t xf[2], wf[4];
@@ -163,8 +166,6 @@ gemm_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const 
         for (int j = 0; j < 4; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[j], xf[i], acc[i][j], 0, 0, 0);
     }
-    if (kt + 1 < nk) stash(buf ^ 1);
-    __syncthreads();
   }
 
   // ---- epilogue: acc element 4*q + r of block (i, j) is row i*32 + l32, column 8*q + 4*(lane/32) + r
@@ -207,7 +208,7 @@ gemm_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const 
 extern "C" SY_API int sy_grouped_gemm(const void* A, const int32_t* a_rows, const void* B, const int32_t* offsets, int E,
                                int rows, int Nout, int K, int swiglu, const void* scale, void* C, void* stream) {
   SY_REQUIRE(rows >= 0 && E >= 1 && Nout >= 1, "grouped_gemm: rows = %d, E = %d, Nout = %d", rows, E, Nout);
-  SY_REQUIRE(K >= BK && K % BK == 0, "grouped_gemm: K must be a multiple of %d (got %d)", BK, K);
+  SY_REQUIRE(K >= 32 && K % 32 == 0, "grouped_gemm: K must be a multiple of 32 (got %d)", K);
   SY_REQUIRE(!(swiglu && scale), "grouped_gemm: swiglu and scale are not combined");
   if (rows == 0) return SY_OK;
   SY_REQUIRE(A && B && offsets && C, "grouped_gemm: null pointer");
