@@ -34,9 +34,10 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published
 EXPERT_BYTES = 3 * H * I * 2   # gate + up + down of one expert, fp16
 T4_WEIGHT_GBS_AT_8 = 232.98490131032196  # the reference's published figure for this metric (Tesla T4)
 
-# HBM bytes per launch of the gate/up projection from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
-# keyed by token count; filled from the summaries under profiles/ (None: not measured).
-MEASURED_TRAFFIC_BYTES = {}
+# HBM bytes per launch of the gate/up projection from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (scaled by a plain copy kernel of known size: 2.0 and 1.0), keyed by token count; the run is
+# summarised in profiles/decode_8tok_gemv_hbm_traffic.txt. Token counts not measured: None.
+MEASURED_TRAFFIC_BYTES = {8: 342.7e6}
 
 
 def make_layers(n_layers, seed=0):
@@ -175,7 +176,7 @@ def run_default(args):
     roof["us_per_launch"] = k_ms * 1e3
     roof["algorithmic_per_launch"] = alg
 
-    cpu = cpu_loop_baseline(h_cpu, *cpu_layers[0], used[0])
+    cpu = None if args.no_cpu else cpu_loop_baseline(h_cpu, *cpu_layers[0], used[0])
 
     line = {
         "metric": "OLMoE MoE-layer expert-weight GB/s", "value": value, "unit": "GB/s", "n_gpus": 1,
@@ -259,12 +260,23 @@ def main():
     ap.add_argument("--layers", type=int, default=4, help="distinct layers' weights to rotate through")
     ap.add_argument("--sweep", default=None, help='"all" or a comma list of token counts')
     ap.add_argument("--no-loops", action="store_true", help="sweep: skip the torch per-expert loops")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="first run a plain 512 MiB device copy 5 times (a kernel of known traffic, to scale "
+                         "rocprofv3's FETCH_SIZE / WRITE_SIZE readings)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg (profiling runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU; --gpus must be 1 (no multi-GPU figure is produced)")
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     with torch.no_grad():
+        if args.calibrate_copy:
+            src = torch.empty(512 << 20, dtype=torch.uint8, device="cuda:0").random_(0, 255)
+            dst = torch.empty_like(src)
+            for _ in range(5):
+                dst.copy_(src)
+            torch.cuda.synchronize()
+            del src, dst
         if args.sweep:
             run_sweep(args)
         else:
