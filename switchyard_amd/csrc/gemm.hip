@@ -88,15 +88,21 @@ gemm_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const 
   const int Nfull = SWIGLU ? 2 * Nout : Nout;
   const half_t* Be = B + (size_t)e * Nfull * K;
 
-  // ---- loader: thread t moves 16-byte chunk (t & 7) of rows (t >> 3) + 32*q
+  // ---- loader: thread t moves 16-byte chunk (t & 7) of rows (t >> 3) + 32*q through buffer
+  // descriptors: a row that does not exist (past the expert's end, past Nout) or a chunk past K
+  // gets an out-of-range offset and reads as 0, so the loop has no branches
   const int lrow = tid >> 3, lch = (tid & 7) * 8;
   constexpr int NA = BM / 32, NB = BW / 32;
-  const half_t* pa[NA];
-  const half_t* pb[NB];
+  constexpr unsigned OUT_OF_RANGE = 0x80000000u;
+  const __amdgpu_buffer_rsrc_t arsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(A), 0, 0x7fffffff, 0x00020000);
+  const __amdgpu_buffer_rsrc_t brsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(Be), 0, (int)((size_t)Nfull * K * 2), 0x00020000);
+  unsigned oa[NA], ob[NB];
 #pragma unroll
   for (int q = 0; q < NA; ++q) {
     const int r = lrow + 32 * q;
-    pa[q] = r < nrows ? A + (size_t)(a_rows ? a_rows[row0 + r] : row0 + r) * K + lch : nullptr;
+    const int src = r < nrows ? (a_rows ? a_rows[row0 + r] : row0 + r) : 0;
+    oa[q] = r < nrows ? ((unsigned)src * (unsigned)K + (unsigned)lch) * 2u : OUT_OF_RANGE;
   }
 #pragma unroll
   for (int q = 0; q < NB; ++q) {
@@ -109,16 +115,17 @@ gemm_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const 
       col = n0 + br;
       wr = col;
     }
-    pb[q] = col < Nout ? Be + (size_t)wr * K + lch : nullptr;
+    ob[q] = col < Nout ? ((unsigned)wr * (unsigned)K + (unsigned)lch) * 2u : OUT_OF_RANGE;
   }
-  const half8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
   half8_t ra[NA], rb[NB];
   auto fetch = [&](int k0) {
     const bool kok = k0 + lch < K;  // K may end in the middle of the last slice
 #pragma unroll
-    for (int q = 0; q < NA; ++q) ra[q] = (pa[q] && kok) ? *reinterpret_cast<const half8_t*>(pa[q] + k0) : zero8;
+    for (int q = 0; q < NA; ++q)
+      ra[q] = __builtin_bit_cast(half8_t, __builtin_amdgcn_raw_buffer_load_b128(arsrc, kok ? oa[q] : OUT_OF_RANGE, k0 * 2, 0));
 #pragma unroll
-    for (int q = 0; q < NB; ++q) rb[q] = (pb[q] && kok) ? *reinterpret_cast<const half8_t*>(pb[q] + k0) : zero8;
+    for (int q = 0; q < NB; ++q)
+      rb[q] = __builtin_bit_cast(half8_t, __builtin_amdgcn_raw_buffer_load_b128(brsrc, kok ? ob[q] : OUT_OF_RANGE, k0 * 2, 0));
   };
   auto stash = [&]() {
     half_t* as = lds;
@@ -210,6 +217,7 @@ extern "C" SY_API int sy_grouped_gemm(const void* A, const int32_t* a_rows, cons
   SY_REQUIRE(rows >= 0 && E >= 1 && Nout >= 1, "grouped_gemm: rows = %d, E = %d, Nout = %d", rows, E, Nout);
   SY_REQUIRE(K >= 32 && K % 32 == 0, "grouped_gemm: K must be a multiple of 32 (got %d)", K);
   SY_REQUIRE(!(swiglu && scale), "grouped_gemm: swiglu and scale are not combined");
+  SY_REQUIRE((long)Nout * K * (swiglu ? 4 : 2) < (1l << 31), "grouped_gemm: an expert's matrix must stay under 2 GiB");
   if (rows == 0) return SY_OK;
   SY_REQUIRE(A && B && offsets && C, "grouped_gemm: null pointer");
   const int cols = swiglu ? BW / 2 : BW;
