@@ -59,6 +59,14 @@ SY_API int sy_sort_by_expert(const int32_t* idx, const void* w, int w_bytes, int
                       int32_t* offsets, int32_t* token, void* wsorted, int32_t* pos_of, void* workspace,
                       size_t workspace_bytes, void* stream);
 
+/* Route and sort of a decode step in ONE launch (one workgroup).
+ * Fuses route() (moe_kernels.cu:73-89) and sort_by_expert() (moe_kernels.cu:142-157), which the
+ * reference's layer calls back to back (switchyard/kernels.py:91-93,84).
+ * logits f16 [N,E] -> exactly the outputs of sy_route (idx, w in f16) and of sy_sort_by_expert.
+ * Limits: 1 <= N <= 256, E <= 128, k <= 8. */
+SY_API int sy_route_sort(const void* logits, int N, int E, int k, int norm, int32_t* idx, void* w, int32_t* counts,
+                         int32_t* offsets, int32_t* token, void* wsorted, int32_t* pos_of, void* stream);
+
 /* Replaces grouped_gemv() (moe_kernels.cu:385-415, kernel :308-383): the decode weight stream.
  * For every expert e and row r in offsets[e]..offsets[e+1]:
  *   C[r,:] = epilogue(A[a_rows ? a_rows[r] : r, :] @ B[e]^T)

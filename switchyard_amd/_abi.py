@@ -26,6 +26,8 @@ SIGNATURES = {
     "sy_sort_workspace_bytes": (_c_size_t, [_c_int, _c_int, _c_int]),
     "sy_sort_by_expert": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p,
                                    _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_size_t, _c_void_p]),
+    "sy_route_sort": (_c_int, [_c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                               _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
     "sy_grouped_gemv": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int,
                                  _c_int, _c_void_p, _c_void_p, _c_void_p]),
     "sy_grouped_gemm": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int,
@@ -107,6 +109,22 @@ class Ext:
                    counts.data_ptr(), offsets.data_ptr(), token.data_ptr(), wsorted.data_ptr(), pos_of.data_ptr(),
                    ws.data_ptr() if need else None, need, _stream())
         return [counts, offsets, token, wsorted, pos_of]
+
+    def route_sort(self, logits, k, norm, n_experts=None):
+        """route then sort_by_expert in one launch (decode). logits [N, E] f16 ->
+        [idx [N, k], w [N, k], counts [E], offsets [E+1], token [M], wsorted [M], pos_of [M]]."""
+        _check(logits, "logits", torch.float16)
+        N, E = logits.shape
+        dev, M = logits.device, N * k
+        i32 = dict(dtype=torch.int32, device=dev)
+        idx, w = torch.empty((N, k), **i32), torch.empty((N, k), dtype=torch.float16, device=dev)
+        counts, offsets = torch.empty(E, **i32), torch.empty(E + 1, **i32)
+        token, pos_of = torch.empty(M, **i32), torch.empty(M, **i32)
+        wsorted = torch.empty(M, dtype=torch.float16, device=dev)
+        self._call(self.lib.sy_route_sort, logits.data_ptr(), N, E, int(k), int(bool(norm)), idx.data_ptr(),
+                   w.data_ptr(), counts.data_ptr(), offsets.data_ptr(), token.data_ptr(), wsorted.data_ptr(),
+                   pos_of.data_ptr(), _stream())
+        return [idx, w, counts, offsets, token, wsorted, pos_of]
 
     def _grouped(self, fn, A, a_rows, B, offsets, rows, swiglu, scale, hint=None):
         _check(A, "A", torch.float16)

@@ -36,17 +36,29 @@ __device__ __forceinline__ float dpp_row_ror(float v) {
   return __int_as_float(dpp_row_ror<N>(__float_as_int(v)));
 }
 
-// All-reduce over the 64 lanes of a wavefront; every lane ends with the same bits because
-// each step combines two values that are themselves identical across the partner lanes.
+// All-reduce inside each row of 16 lanes with DPP rotations: every lane of a row ends with the
+// same bits, because each step combines two values that are identical across partner lanes.
 template <typename T, typename Op>
-__device__ __forceinline__ T wave_allreduce(T v, Op op) {
+__device__ __forceinline__ T row_allreduce(T v, Op op) {
   v = op(v, dpp_row_ror<8>(v));
   v = op(v, dpp_row_ror<4>(v));
   v = op(v, dpp_row_ror<2>(v));
   v = op(v, dpp_row_ror<1>(v));
-  v = op(v, __shfl_xor(v, 16, WAVE));
-  v = op(v, __shfl_xor(v, 32, WAVE));
   return v;
+}
+
+__device__ __forceinline__ float read_lane(float v, int lane) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+__device__ __forceinline__ int read_lane(int v, int lane) { return __builtin_amdgcn_readlane(v, lane); }
+
+// All-reduce over the 64 lanes of a wavefront: DPP inside the four rows, then the four row
+// results are read into scalar registers and combined in a fixed order, so the result is
+// wave-uniform and needs no trip through the LDS crossbar.
+template <typename T, typename Op>
+__device__ __forceinline__ T wave_allreduce(T v, Op op) {
+  v = row_allreduce(v, op);
+  return op(op(read_lane(v, 0), read_lane(v, 16)), op(read_lane(v, 32), read_lane(v, 48)));
 }
 
 __device__ __forceinline__ float wave_max(float v) {

@@ -96,6 +96,20 @@ def experts(h, idx, w, gate_up, down, mode="auto"):
     return E.combine(y, pos_of, idx, N)
 
 
+# Up to this many tokens route and sort run as one launch of one workgroup (a decode step is
+# launch- and latency-bound in front of its two projections).
+FUSED_FRONT_MAX_TOKENS = 64
+
+
 def moe_layer(h, router, gate_up, down, top_k, norm_topk_prob, mode="auto"):
+    N, n_experts = h.shape[0], gate_up.shape[0]
+    if 0 < N <= FUSED_FRONT_MAX_TOKENS and n_experts <= 128 and top_k <= 8 and h.dtype == torch.float16:
+        E = ext()
+        idx, w, counts, offsets, token, wsorted, pos_of = E.route_sort(F.linear(h, router).contiguous(), top_k,
+                                                                       norm_topk_prob)
+        if mode == "auto":
+            mode = _auto(N, idx.numel(), n_experts)
+        y = ffn(h, token, offsets, counts, wsorted, gate_up, down, idx.numel(), mode)
+        return E.combine(y, pos_of, idx, N)
     idx, w = route(h, router, top_k, norm_topk_prob)
     return experts(h, idx, w, gate_up, down, mode)

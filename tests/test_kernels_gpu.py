@@ -311,3 +311,34 @@ def test_full_size_properties(K, olmoe, N, mode):
     assert torch.allclose(doubled.float(), 2 * out.float(), rtol=2.0 ** -10, atol=2.0 ** -23)
     other = K.experts(h, idx, w, gu, dn, "gemm" if mode == "gemv" else "gemv")
     assert (other.float() - out.float()).abs().max().item() < 2e-3
+
+
+# ------------------------------------------------------------------ route + sort in one launch (decode)
+@pytest.mark.parametrize("N,E,k,H", [(1, 64, 8, 2048), (8, 64, 8, 2048), (33, 64, 8, 2048), (64, 64, 8, 256),
+                                     (256, 64, 8, 256), (7, 128, 8, 512), (20, 16, 4, 128), (5, 60, 3, 64)])
+@pytest.mark.parametrize("norm", [False, True])
+def test_route_sort_in_one_launch(K, N, E, k, H, norm):
+    """Bit for bit what route followed by sort_by_expert gives, and what the oracle gives."""
+    g = torch.Generator().manual_seed(N * 7 + E)
+    h = torch.randn(N, H, generator=g).half().to(DEV)
+    router = (torch.randn(E, H, generator=g) * H ** -0.5).half().to(DEV)
+    logits = F.linear(h, router).contiguous()
+    idx, w, counts, offsets, token, wsorted, pos_of = K.ext().route_sort(logits, k, norm)
+    ridx, rw = K.ext().route(logits, k, norm)
+    assert torch.equal(idx, ridx) and torch.equal(w, rw)
+    for a, b in zip((counts, offsets, token, wsorted, pos_of), K.ext().sort_by_expert(ridx, rw, E)):
+        assert torch.equal(a, b)
+    oidx, ow = O.route_logits(logits.cpu(), k, norm)
+    assert torch.equal(idx.cpu().long(), oidx)
+    assert (w.cpu().float() - ow.float()).abs().max().item() < WEIGHT_TOL
+    p = O.plan(oidx, w.cpu(), E)
+    assert torch.equal(counts.cpu().long(), p.counts) and torch.equal(offsets.cpu().long(), p.offsets)
+    assert torch.equal(token.cpu().long(), p.token) and torch.equal(pos_of.cpu().long(), p.pos_of)
+    assert torch.equal(wsorted.cpu().view(torch.int16), p.weight.view(torch.int16))
+
+
+def test_route_sort_limits(K):
+    with pytest.raises(RuntimeError):
+        K.ext().route_sort(torch.zeros(300, 64, dtype=torch.float16, device=DEV), 8, False)   # too many tokens
+    with pytest.raises(RuntimeError):
+        K.ext().route_sort(torch.zeros(4, 64, dtype=torch.float16, device=DEV), 9, False)
