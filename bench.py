@@ -250,6 +250,69 @@ def run_sweep(args):
         print(json.dumps(rec), flush=True)
 
 
+def run_decode(args):
+    """Full OLMoE-1B-7B-shaped model (16 layers, random-init fp16, ~14 GB), greedy decode of
+    `--new-tokens` tokens from random prompts of `--prompt-len` tokens; attention in PyTorch,
+    MoE layers through the hook. One JSON line per batch size."""
+    from oracle import moe_oracle as O
+    from switchyard_amd import decoder as D
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    s = D.OLMOE_1B_7B
+    w = D.random_weights(s, device=dev, seed=0)
+    model = D.Decoder(s, w, max_positions=args.prompt_len + args.new_tokens + 8)
+
+    def loop_moe(i, h):
+        L = w["layers"][i]
+        return O.moe_layer(h, L["router"], L["gate_up"], L["down"], s.top_k, s.norm_topk_prob)
+
+    loop_model = D.Decoder(s, w, moe=loop_moe, max_positions=args.prompt_len + args.new_tokens + 8)
+    for B in [int(x) for x in args.decode.split(",")]:
+        g = torch.Generator().manual_seed(0)
+        prompts = torch.randint(3, s.vocab, (B, args.prompt_len), generator=g).tolist()
+        tokens = torch.tensor(prompts, device=dev)
+        # one untimed generation warms every kernel; then the decode step is captured in a HIP
+        # graph and replayed once per token (prefill and replay loop timed separately)
+        model.generate(prompts, 4)
+        torch.cuda.synchronize()
+        tm = {}
+        graph_tokens, first = model.generate_graph(prompts, args.new_tokens + 1, return_first_logits=True, timings=tm)
+        t_prefill, t_decode, steps = tm["prefill_s"], tm["decode_s"], tm["decode_steps"]
+        # the eager loop (one Python-driven step per token) for comparison, fewer tokens
+        cache = D.KVCache(s, B, args.prompt_len + 16, torch.float16, dev)
+        logits = model.forward(tokens, cache)[:, -1]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(16):
+            logits = model.forward(logits.argmax(-1)[:, None], cache)[:, -1]
+        torch.cuda.synchronize()
+        t_eager = (time.perf_counter() - t0) / 16
+        # the same prompts through the per-expert loop hook: first-token logits must agree on the top-1
+        ref_first = loop_model.forward(tokens)[:, -1]
+        agree = first.argmax(-1) == ref_first.argmax(-1)
+        top2 = ref_first.float().topk(2, dim=-1).values
+        margin = (top2[:, 0] - top2[:, 1])
+        rec = {"bench": "decode", "batch": B, "prompt_len": args.prompt_len, "new_tokens": steps,
+               "decode_tok_per_s": B * steps / t_decode, "ms_per_step": t_decode * 1e3 / steps,
+               "eager_ms_per_step": t_eager * 1e3, "eager_decode_tok_per_s": B / t_eager,
+               "prefill_tok_per_s": B * args.prompt_len / t_prefill, "prefill_ms": t_prefill * 1e3,
+               "top1_rows_identical_to_loop_hook": int(agree.sum()), "rows": B,
+               "largest_loop_hook_margin_where_top1_differs": float(margin[~agree].max()) if (~agree).any() else 0.0,
+               "first_logits_max_abs_diff": (first.float() - ref_first.float()).abs().max().item(),
+               "model": "OLMoE-1B-7B shape, 16 layers, random-init fp16", "gpu": torch.cuda.get_device_name(0)}
+        if args.decode_loop_steps:
+            cache = D.KVCache(s, B, args.prompt_len + args.decode_loop_steps, torch.float16, dev)
+            logits = loop_model.forward(tokens, cache)[:, -1]
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.decode_loop_steps):
+                logits = loop_model.forward(logits.argmax(-1)[:, None], cache)[:, -1]
+            torch.cuda.synchronize()
+            rec["loop_hook_decode_tok_per_s"] = B * args.decode_loop_steps / (time.perf_counter() - t0)
+        print(json.dumps(rec), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -264,6 +327,11 @@ def main():
                     help="first run a plain 512 MiB device copy 5 times (a kernel of known traffic, to scale "
                          "rocprofv3's FETCH_SIZE / WRITE_SIZE readings)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg (profiling runs)")
+    ap.add_argument("--decode", default=None, help='full-model greedy decode at these batch sizes, e.g. "8,64"')
+    ap.add_argument("--prompt-len", type=int, default=512)
+    ap.add_argument("--new-tokens", type=int, default=128)
+    ap.add_argument("--decode-loop-steps", type=int, default=8,
+                    help="decode steps to time with the per-expert loop in the hook (0: skip)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU; --gpus must be 1 (no multi-GPU figure is produced)")
@@ -277,7 +345,9 @@ def main():
                 dst.copy_(src)
             torch.cuda.synchronize()
             del src, dst
-        if args.sweep:
+        if args.decode:
+            run_decode(args)
+        elif args.sweep:
             run_sweep(args)
         else:
             run_default(args)

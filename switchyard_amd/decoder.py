@@ -1,0 +1,334 @@
+"""An OLMoE decoder around the MoE layer: the caller of the hot path.
+
+Counterpart of the reference's switchyard/model.py (the `self.moe(i, h)` hook at :39-42,135)
+and of the tensor layout its weights.py defines (:36-69). Attention stays in PyTorch; every
+mixture-of-experts layer goes through `moe(layer_index, h[B*T, H]) -> [B*T, H]`, which by
+default is `kernels.moe_layer` on the layer's router / gate_up / down tensors.
+
+Built for decode on one GPU: the KV cache is allocated once for the whole generation, rotary
+tables are precomputed, attention is one fused scaled-dot-product call, and the greedy loop
+keeps its tokens on the device, so a decode step is a queue of launches with no host read
+unless the caller asks for early stopping at `eos`.
+"""
+
+from dataclasses import dataclass
+
+import torch
+import torch.nn.functional as F
+
+
+@dataclass
+class Shape:
+    vocab: int = 50304
+    hidden: int = 2048
+    intermediate: int = 1024       # per expert
+    layers: int = 16
+    heads: int = 16
+    kv_heads: int = 16
+    head_dim: int = 128
+    experts: int = 64
+    top_k: int = 8
+    norm_topk_prob: bool = False
+    rms_eps: float = 1e-5
+    rope_theta: float = 10000.0
+    clip_qkv: float | None = None
+
+    @classmethod
+    def from_hf(cls, c):
+        """From a transformers OlmoeConfig (or any object with its attribute names)."""
+        heads = c.num_attention_heads
+        rope = getattr(c, "rope_parameters", None) or {}
+        return cls(vocab=c.vocab_size, hidden=c.hidden_size, intermediate=c.intermediate_size,
+                   layers=c.num_hidden_layers, heads=heads, kv_heads=getattr(c, "num_key_value_heads", None) or heads,
+                   head_dim=getattr(c, "head_dim", None) or c.hidden_size // heads, experts=c.num_experts,
+                   top_k=c.num_experts_per_tok, norm_topk_prob=bool(getattr(c, "norm_topk_prob", False)),
+                   rms_eps=getattr(c, "rms_norm_eps", 1e-5),
+                   rope_theta=rope.get("rope_theta", getattr(c, "rope_theta", 10000.0)),
+                   clip_qkv=getattr(c, "clip_qkv", None))
+
+
+OLMOE_1B_7B = Shape()
+
+
+def random_weights(shape, dtype=torch.float16, device="cuda", seed=0, std=0.02):
+    """Random-initialised weights in the layout the reference's loader produces: experts stacked
+    as gate_up [E, 2I, H] (gate rows first) and down [E, H, I]; norm weights 1."""
+    g = torch.Generator(device=device).manual_seed(seed)
+
+    def rnd(*dims):
+        return (torch.randn(*dims, generator=g, device=device, dtype=torch.float32) * std).to(dtype)
+
+    s = shape
+    qd, kvd = s.heads * s.head_dim, s.kv_heads * s.head_dim
+    layers = []
+    for _ in range(s.layers):
+        layers.append(dict(
+            attn_norm=torch.ones(s.hidden, dtype=dtype, device=device),
+            wq=rnd(qd, s.hidden), wk=rnd(kvd, s.hidden), wv=rnd(kvd, s.hidden), wo=rnd(s.hidden, qd),
+            q_norm=torch.ones(qd, dtype=dtype, device=device), k_norm=torch.ones(kvd, dtype=dtype, device=device),
+            mlp_norm=torch.ones(s.hidden, dtype=dtype, device=device),
+            router=rnd(s.experts, s.hidden), gate_up=rnd(s.experts, 2 * s.intermediate, s.hidden),
+            down=rnd(s.experts, s.hidden, s.intermediate)))
+    return dict(embed=rnd(s.vocab, s.hidden), final_norm=torch.ones(s.hidden, dtype=dtype, device=device),
+                lm_head=rnd(s.vocab, s.hidden), layers=layers)
+
+
+def weights_from_hf(state_dict, shape, dtype=None, device=None):
+    """The same layout from a transformers OlmoeForCausalLM state dict (stacked or per-expert names)."""
+    def get(name):
+        t = state_dict[name]
+        return t.to(dtype=dtype or t.dtype, device=device or t.device).contiguous()
+
+    layers = []
+    for i in range(shape.layers):
+        p = f"model.layers.{i}."
+        if p + "mlp.experts.gate_up_proj" in state_dict:
+            gate_up, down = get(p + "mlp.experts.gate_up_proj"), get(p + "mlp.experts.down_proj")
+        else:
+            gate_up = torch.stack([torch.cat([get(f"{p}mlp.experts.{e}.gate_proj.weight"),
+                                              get(f"{p}mlp.experts.{e}.up_proj.weight")]) for e in range(shape.experts)])
+            down = torch.stack([get(f"{p}mlp.experts.{e}.down_proj.weight") for e in range(shape.experts)])
+        layers.append(dict(
+            attn_norm=get(p + "input_layernorm.weight"), mlp_norm=get(p + "post_attention_layernorm.weight"),
+            wq=get(p + "self_attn.q_proj.weight"), wk=get(p + "self_attn.k_proj.weight"),
+            wv=get(p + "self_attn.v_proj.weight"), wo=get(p + "self_attn.o_proj.weight"),
+            q_norm=get(p + "self_attn.q_norm.weight"), k_norm=get(p + "self_attn.k_norm.weight"),
+            router=get(p + "mlp.gate.weight"), gate_up=gate_up, down=down))
+    lm_head = get("lm_head.weight") if "lm_head.weight" in state_dict else get("model.embed_tokens.weight")
+    return dict(embed=get("model.embed_tokens.weight"), final_norm=get("model.norm.weight"), lm_head=lm_head,
+                layers=layers)
+
+
+def _rms(x, weight, eps):
+    # normalise in fp32, cast back, then scale: the order transformers uses
+    f = x.float()
+    return weight * (f * torch.rsqrt(f.square().mean(-1, keepdim=True) + eps)).to(x.dtype)
+
+
+def _rotate(x, cos, sin):
+    half = x.shape[-1] // 2
+    return x * cos + torch.cat([-x[..., half:], x[..., :half]], dim=-1) * sin
+
+
+class KVCache:
+    """Keys and values of every layer, [B, kv_heads, capacity, head_dim], allocated once.
+    `filled` positions are in use; `real[b, p]` is False where batch row b holds left padding."""
+
+    def __init__(self, shape, batch, capacity, dtype, device):
+        dims = (shape.layers, batch, shape.kv_heads, capacity, shape.head_dim)
+        self.k = torch.zeros(dims, dtype=dtype, device=device)
+        self.v = torch.zeros(dims, dtype=dtype, device=device)
+        self.real = torch.zeros(batch, capacity, dtype=torch.bool, device=device)
+        self.next_position = torch.zeros(batch, dtype=torch.long, device=device)
+        self.filled = 0
+        self.capacity = capacity
+
+
+class Decoder:
+    def __init__(self, shape, weights, moe=None, max_positions=4096):
+        self.s, self.w = shape, weights
+        self.moe = moe or self.kernel_moe
+        dev = weights["embed"].device
+        inv = 1.0 / (shape.rope_theta ** (torch.arange(0, shape.head_dim, 2, device=dev).float() / shape.head_dim))
+        ang = torch.outer(torch.arange(max_positions, device=dev).float(), inv)
+        table = torch.cat([ang, ang], dim=-1)
+        self.cos, self.sin = table.cos().to(weights["embed"].dtype), table.sin().to(weights["embed"].dtype)
+
+    # ---- the hook's default: the gfx950 kernels
+    def kernel_moe(self, i, h):
+        from . import kernels
+
+        L = self.w["layers"][i]
+        return kernels.moe_layer(h, L["router"], L["gate_up"], L["down"], self.s.top_k, self.s.norm_topk_prob)
+
+    def _attend(self, i, x, positions, mask, cache, start):
+        s, L = self.s, self.w["layers"][i]
+        B, T, _ = x.shape
+        q = _rms(F.linear(x, L["wq"]), L["q_norm"], s.rms_eps)
+        k = _rms(F.linear(x, L["wk"]), L["k_norm"], s.rms_eps)
+        v = F.linear(x, L["wv"])
+        if s.clip_qkv is not None:
+            q, k, v = q.clamp(-s.clip_qkv, s.clip_qkv), k.clamp(-s.clip_qkv, s.clip_qkv), v.clamp(-s.clip_qkv, s.clip_qkv)
+        q = q.view(B, T, s.heads, s.head_dim).transpose(1, 2)
+        k = k.view(B, T, s.kv_heads, s.head_dim).transpose(1, 2)
+        v = v.view(B, T, s.kv_heads, s.head_dim).transpose(1, 2)
+        cos, sin = self.cos[positions][:, None], self.sin[positions][:, None]
+        q, k = _rotate(q, cos, sin), _rotate(k, cos, sin)
+        if cache is not None:
+            cache.k[i, :, :, start:start + T] = k
+            cache.v[i, :, :, start:start + T] = v
+            k, v = cache.k[i, :, :, :start + T], cache.v[i, :, :, :start + T]
+        a = F.scaled_dot_product_attention(q, k, v, attn_mask=mask, enable_gqa=s.kv_heads != s.heads)
+        return F.linear(a.transpose(1, 2).reshape(B, T, s.heads * s.head_dim), L["wo"])
+
+    @torch.no_grad()
+    def forward(self, tokens, cache=None, valid=None):
+        """tokens [B, T] -> logits [B, T, vocab]. `valid` [B, T] marks real tokens (False = left
+        padding). With a cache the tokens are appended after what it already holds."""
+        s, W = self.s, self.w
+        B, T = tokens.shape
+        dev = tokens.device
+        if valid is None:
+            valid = torch.ones(B, T, dtype=torch.bool, device=dev)
+        start = cache.filled if cache is not None else 0
+        base = cache.next_position if cache is not None else torch.zeros(B, dtype=torch.long, device=dev)
+        positions = (base[:, None] + valid.long().cumsum(1) - 1).clamp_(min=0)
+        if cache is not None:
+            cache.real[:, start:start + T] = valid
+            keys_real = cache.real[:, :start + T]
+        else:
+            keys_real = valid
+        # query q (absolute index start+q) sees key j <= start+q that holds a real token; a padding
+        # query would see nothing, so it is allowed itself (its output is never used)
+        qi = torch.arange(start, start + T, device=dev)[:, None]
+        kj = torch.arange(start + T, device=dev)[None, :]
+        mask = (kj <= qi)[None] & keys_real[:, None, :]
+        mask = mask | ((kj == qi)[None] & ~mask.any(-1, keepdim=True))
+        mask = mask[:, None]  # broadcast over heads
+
+        x = F.embedding(tokens, W["embed"])
+        for i in range(s.layers):
+            L = W["layers"][i]
+            x = x + self._attend(i, _rms(x, L["attn_norm"], s.rms_eps), positions, mask, cache, start)
+            h = _rms(x, L["mlp_norm"], s.rms_eps).reshape(B * T, s.hidden)
+            x = x + self.moe(i, h).view(B, T, s.hidden)
+        if cache is not None:
+            cache.filled = start + T
+            cache.next_position = base + valid.long().sum(1)
+        return F.linear(_rms(x, W["final_norm"], s.rms_eps), W["lm_head"])
+
+    # ---- one decode step with every index on the device, so that it can be captured in a HIP graph
+    @torch.no_grad()
+    def step_static(self, tok, cache, slot, keys):
+        """tok [B, 1] -> logits [B, vocab]. `slot` is a one-element device tensor holding the cache
+        position to write (the same for every row of a left-padded batch); `keys` is
+        arange(capacity). Attention runs over the whole capacity under a mask, shapes never change,
+        and nothing depends on a host value: the step is a fixed sequence of launches."""
+        s, W = self.s, self.w
+        B = tok.shape[0]
+        positions = cache.next_position[:, None]
+        cache.real.index_fill_(1, slot, True)
+        mask = ((keys[None, :] <= slot) & cache.real)[:, None, None, :]
+        x = F.embedding(tok, W["embed"])
+        for i in range(s.layers):
+            L = W["layers"][i]
+            xn = _rms(x, L["attn_norm"], s.rms_eps)
+            q = _rms(F.linear(xn, L["wq"]), L["q_norm"], s.rms_eps)
+            k = _rms(F.linear(xn, L["wk"]), L["k_norm"], s.rms_eps)
+            v = F.linear(xn, L["wv"])
+            if s.clip_qkv is not None:
+                q, k, v = (q.clamp(-s.clip_qkv, s.clip_qkv), k.clamp(-s.clip_qkv, s.clip_qkv),
+                           v.clamp(-s.clip_qkv, s.clip_qkv))
+            q = q.view(B, 1, s.heads, s.head_dim).transpose(1, 2)
+            k = k.view(B, 1, s.kv_heads, s.head_dim).transpose(1, 2)
+            v = v.view(B, 1, s.kv_heads, s.head_dim).transpose(1, 2)
+            cos, sin = self.cos[positions][:, None], self.sin[positions][:, None]
+            q, k = _rotate(q, cos, sin), _rotate(k, cos, sin)
+            cache.k[i].index_copy_(2, slot, k)
+            cache.v[i].index_copy_(2, slot, v)
+            a = F.scaled_dot_product_attention(q, cache.k[i], cache.v[i], attn_mask=mask,
+                                               enable_gqa=s.kv_heads != s.heads)
+            x = x + F.linear(a.transpose(1, 2).reshape(B, 1, s.heads * s.head_dim), L["wo"])
+            h = _rms(x, L["mlp_norm"], s.rms_eps).reshape(B, s.hidden)
+            x = x + self.moe(i, h).view(B, 1, s.hidden)
+        cache.next_position += 1
+        slot += 1
+        return F.linear(_rms(x, W["final_norm"], s.rms_eps), W["lm_head"])[:, -1]
+
+    @torch.no_grad()
+    def generate_graph(self, prompts, max_new_tokens, return_first_logits=False, timings=None):
+        """Greedy decoding with the decode step captured once in a HIP graph and replayed per
+        token: prefill eagerly, then one graph launch per generated token and no host work in
+        between (no early stop at an eos token). Same tokens as `generate`. If `timings` is a
+        dict, the wall times of the prefill and of the replay loop are stored in it (this adds two
+        device synchronisations)."""
+        import time
+        dev, dtype = self.w["embed"].device, self.w["embed"].dtype
+        B, P = len(prompts), max(len(p) for p in prompts)
+        tokens = torch.zeros(B, P, dtype=torch.long)
+        valid = torch.zeros(B, P, dtype=torch.bool)
+        for b, p in enumerate(prompts):
+            tokens[b, P - len(p):] = torch.tensor(p, dtype=torch.long)
+            valid[b, P - len(p):] = True
+        cache = KVCache(self.s, B, P + max_new_tokens, dtype, dev)
+        tokens, valid = tokens.to(dev), valid.to(dev)
+        if timings is not None:
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+        first_logits = self.forward(tokens, cache, valid)[:, -1]
+        if timings is not None:
+            torch.cuda.synchronize()
+            timings["prefill_s"] = time.perf_counter() - t0
+        out = torch.zeros(B, max_new_tokens, dtype=torch.long, device=dev)
+        tok = first_logits.argmax(-1)[:, None].clone()
+        out[:, 0] = tok[:, 0]
+        if max_new_tokens > 1:
+            slot = torch.tensor([cache.filled], dtype=torch.long, device=dev)
+            col = torch.ones(1, dtype=torch.long, device=dev)       # column of `out` the next token goes to
+            keys = torch.arange(cache.capacity, device=dev)
+
+            def one_token():
+                logits = self.step_static(tok, cache, slot, keys)
+                tok.copy_(logits.argmax(-1)[:, None])
+                out.index_copy_(1, col, tok)
+                col.add_(1)
+
+            # warm up on a side stream (allocator, kernel loading), then restore the state it touched
+            saved = (cache.next_position.clone(), slot.clone(), col.clone(), tok.clone(), cache.real.clone())
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                one_token()
+            torch.cuda.current_stream().wait_stream(side)
+            cache.next_position.copy_(saved[0]); slot.copy_(saved[1]); col.copy_(saved[2]); tok.copy_(saved[3])
+            cache.real.copy_(saved[4])
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                one_token()
+            cache.next_position.copy_(saved[0]); slot.copy_(saved[1]); col.copy_(saved[2]); tok.copy_(saved[3])
+            cache.real.copy_(saved[4])
+            if timings is not None:
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+            for _ in range(max_new_tokens - 1):
+                graph.replay()
+            if timings is not None:
+                torch.cuda.synchronize()
+                timings["decode_s"] = time.perf_counter() - t0
+                timings["decode_steps"] = max_new_tokens - 1
+        rows = out.tolist()
+        return (rows, first_logits) if return_first_logits else rows
+
+    @torch.no_grad()
+    def generate(self, prompts, max_new_tokens, eos=None, return_first_logits=False):
+        """Greedy decoding of a batch of token lists, left-padded internally. Returns the generated
+        tokens of each prompt (cut after `eos` if given). Without `eos` nothing is read back from
+        the device until the end."""
+        dev, dtype = self.w["embed"].device, self.w["embed"].dtype
+        B, P = len(prompts), max(len(p) for p in prompts)
+        tokens = torch.zeros(B, P, dtype=torch.long)
+        valid = torch.zeros(B, P, dtype=torch.bool)
+        for b, p in enumerate(prompts):
+            tokens[b, P - len(p):] = torch.tensor(p, dtype=torch.long)
+            valid[b, P - len(p):] = True
+        tokens, valid = tokens.to(dev), valid.to(dev)
+        cache = KVCache(self.s, B, P + max_new_tokens, dtype, dev)
+        logits = self.forward(tokens, cache, valid)[:, -1]
+        first_logits = logits
+        out = torch.empty(B, max_new_tokens, dtype=torch.long, device=dev)
+        steps = 0
+        alive = torch.ones(B, dtype=torch.bool, device=dev)
+        for step in range(max_new_tokens):
+            nxt = logits.argmax(-1)
+            out[:, step] = nxt
+            steps = step + 1
+            if eos is not None:
+                alive &= nxt != eos
+                if not bool(alive.any()):
+                    break
+            if step + 1 < max_new_tokens:
+                logits = self.forward(nxt[:, None], cache)[:, -1]
+        rows = out[:, :steps].tolist()
+        if eos is not None:
+            rows = [r[:r.index(eos) + 1] if eos in r else r for r in rows]
+        return (rows, first_logits) if return_first_logits else rows
