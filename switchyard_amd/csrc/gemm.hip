@@ -1,8 +1,8 @@
 // grouped_gemm: the prefill path. Every expert's slice of the sorted rows goes through that
 // expert's weights on fp16 MFMA tiles, all experts in one launch.
 //
-// Tile: 128 rows x 256 weight rows, K in slices of 64, 4 wavefronts (2 x 2), each computing
-// 64 rows x 128 weight rows as 2 x 4 v_mfma_f32_32x32x16_f16 blocks with fp32 accumulators.
+// Tile: 64*MI rows x 256 weight rows (MI = 1 or 2), K in slices of 64, 4 wavefronts (2 x 2), each
+// computing 32*MI rows x 128 weight rows as MI x 4 v_mfma_f32_32x32x16_f16 blocks with fp32 accumulators.
 // With SwiGLU the 256 weight rows are 128 gate rows and the 128 up rows of the same output
 // columns, and a wavefront holds gate and up of the same 64 columns, so the activation is
 // applied in registers. Weights are the MFMA M operand and rows the N operand: a lane ends
@@ -28,7 +28,6 @@
 
 namespace {
 
-constexpr int BM = 128;          // rows per tile
 constexpr int BW = 256;          // weight rows per tile
 constexpr int BK = 64;           // K per slice
 constexpr int LDS_LD = BK + 8;   // halves per LDS row (144 bytes)
@@ -41,11 +40,12 @@ __device__ __forceinline__ half_t swiglu_f16(float gate, float up) {
   return (half_t)(s * u);
 }
 
-template <bool SWIGLU, bool SCALE>
+template <int MI, bool SWIGLU, bool SCALE>
 __global__ void __launch_bounds__(GEMM_THREADS, 2)
 gemm_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const half_t* __restrict__ B,
             const int* __restrict__ offsets, int E, int Nout, int K, const half_t* __restrict__ scale,
             half_t* __restrict__ C, int ncol_tiles, int per_xcd) {
+  constexpr int BM = 64 * MI;  // rows per tile
   __shared__ __attribute__((aligned(16))) half_t lds[(BM + BW) * LDS_LD];
   __shared__ int s_tile[3];
 
@@ -143,9 +143,9 @@ gemm_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const 
 #pragma unroll
   for (int j = 0; j < 4; ++j) brow[j] = SWIGLU ? (j >> 1) * COLS + wn * 64 + (j & 1) * 32 : wn * 128 + j * 32;
 
-  float16_t acc[2][4];
+  float16_t acc[MI][4];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < MI; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -153,7 +153,7 @@ gemm_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const 
 
   fetch(0);
   const int nk = (K + BK - 1) / BK;
-  const half_t* as = lds + (wm * 64 + l32) * LDS_LD + lk;
+  const half_t* as = lds + (wm * 32 * MI + l32) * LDS_LD + lk;
   const half_t* bs = lds + (BM + l32) * LDS_LD + lk;
   for (int kt = 0; kt < nk; ++kt) {
     if (kt) __syncthreads();  // every wavefront is done reading the previous slice
@@ -162,13 +162,13 @@ gemm_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const 
     if (kt + 1 < nk) fetch((kt + 1) * BK);
 #pragma unroll
     for (int kk = 0; kk < BK; kk += 16) {
-      half8_t xf[2], wf[4];
+      half8_t xf[MI], wf[4];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) xf[i] = *reinterpret_cast<const half8_t*>(as + i * 32 * LDS_LD + kk);
+      for (int i = 0; i < MI; ++i) xf[i] = *reinterpret_cast<const half8_t*>(as + i * 32 * LDS_LD + kk);
 #pragma unroll
       for (int j = 0; j < 4; ++j) wf[j] = *reinterpret_cast<const half8_t*>(bs + brow[j] * LDS_LD + kk);
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[j], xf[i], acc[i][j], 0, 0, 0);
@@ -178,8 +178,8 @@ gemm_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const 
   // ---- epilogue: acc element 4*q + r of block (i, j) is row i*32 + l32, column 8*q + 4*(lane/32) + r
   const int chalf = (lane >> 5) * 4;
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int row = row0 + wm * 64 + i * 32 + l32;
+  for (int i = 0; i < MI; ++i) {
+    const int row = row0 + wm * 32 * MI + i * 32 + l32;
     if (row >= row_end) continue;
     const float sc_row = SCALE ? (float)scale[row] : 1.f;
     half_t* crow = C + (size_t)row * Nout;
@@ -210,6 +210,27 @@ gemm_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const 
   }
 }
 
+template <int MI>
+int launch_gemm(const half_t* a, const int32_t* a_rows, const half_t* b, const int32_t* offsets, int E, int rows,
+                int Nout, int K, int swiglu, const half_t* s, half_t* c, hipStream_t st) {
+  constexpr int BM = 64 * MI;
+  const int cols = swiglu ? BW / 2 : BW;
+  const int ncol_tiles = (Nout + cols - 1) / cols;
+  // sum over experts of ceil(count / BM) <= rows / BM + (experts with rows) <= rows / BM + min(E, rows)
+  const long max_row_tiles = rows / BM + (E < rows ? E : rows);
+  const long total = max_row_tiles * ncol_tiles;
+  if (total >= (1l << 31) - XCDS) return sy_fail(SY_ERR_ARG, "grouped_gemm: too many tiles");
+  const int per_xcd = (int)((total + XCDS - 1) / XCDS);
+  const int grid = per_xcd * XCDS;
+  if (swiglu)
+    gemm_kernel<MI, true, false><<<grid, GEMM_THREADS, 0, st>>>(a, a_rows, b, offsets, E, Nout, K, nullptr, c, ncol_tiles, per_xcd);
+  else if (s)
+    gemm_kernel<MI, false, true><<<grid, GEMM_THREADS, 0, st>>>(a, a_rows, b, offsets, E, Nout, K, s, c, ncol_tiles, per_xcd);
+  else
+    gemm_kernel<MI, false, false><<<grid, GEMM_THREADS, 0, st>>>(a, a_rows, b, offsets, E, Nout, K, nullptr, c, ncol_tiles, per_xcd);
+  return sy_check_launch("grouped_gemm");
+}
+
 }  // namespace
 
 extern "C" SY_API int sy_grouped_gemm(const void* A, const int32_t* a_rows, const void* B, const int32_t* offsets, int E,
@@ -220,24 +241,16 @@ extern "C" SY_API int sy_grouped_gemm(const void* A, const int32_t* a_rows, cons
   SY_REQUIRE((long)Nout * K * (swiglu ? 4 : 2) < (1l << 31), "grouped_gemm: an expert's matrix must stay under 2 GiB");
   if (rows == 0) return SY_OK;
   SY_REQUIRE(A && B && offsets && C, "grouped_gemm: null pointer");
-  const int cols = swiglu ? BW / 2 : BW;
-  const int ncol_tiles = (Nout + cols - 1) / cols;
-  // sum over experts of ceil(count / BM) <= rows / BM + (experts with rows) <= rows / BM + min(E, rows)
-  const long max_row_tiles = rows / BM + (E < rows ? E : rows);
-  const long total = max_row_tiles * ncol_tiles;
-  SY_REQUIRE(total < (1l << 31) - XCDS, "grouped_gemm: too many tiles");
-  const int per_xcd = (int)((total + XCDS - 1) / XCDS);
-  const int grid = per_xcd * XCDS;
-  hipStream_t st = (hipStream_t)stream;
+  // rows per tile: 64 while the typical expert fits in one such tile (the launch is then a
+  // stream over the weights and the smaller tile halves the padded MFMA work), else 128. Under
+  // near-uniform routing an expert's rows scatter around the mean by about its square root.
+  const int mean = (rows + E - 1) / E;
+  int typical = mean;
+  while ((typical - mean) * (typical - mean) < 4 * mean) ++typical;
   const half_t* a = (const half_t*)A;
   const half_t* b = (const half_t*)B;
   const half_t* s = (const half_t*)scale;
   half_t* c = (half_t*)C;
-  if (swiglu)
-    gemm_kernel<true, false><<<grid, GEMM_THREADS, 0, st>>>(a, a_rows, b, offsets, E, Nout, K, nullptr, c, ncol_tiles, per_xcd);
-  else if (s)
-    gemm_kernel<false, true><<<grid, GEMM_THREADS, 0, st>>>(a, a_rows, b, offsets, E, Nout, K, s, c, ncol_tiles, per_xcd);
-  else
-    gemm_kernel<false, false><<<grid, GEMM_THREADS, 0, st>>>(a, a_rows, b, offsets, E, Nout, K, nullptr, c, ncol_tiles, per_xcd);
-  return sy_check_launch("grouped_gemm");
+  if (typical <= 64) return launch_gemm<1>(a, a_rows, b, offsets, E, rows, Nout, K, swiglu, s, c, (hipStream_t)stream);
+  return launch_gemm<2>(a, a_rows, b, offsets, E, rows, Nout, K, swiglu, s, c, (hipStream_t)stream);
 }

@@ -13,6 +13,8 @@ Differences that follow from the hardware, none visible in the results:
     "cublas" is still accepted and runs the MFMA kernel.
 """
 
+import math
+
 import torch
 import torch.nn.functional as F
 
@@ -40,9 +42,10 @@ def route(h, router, top_k, norm_topk_prob):
     return ext().route(F.linear(h, router).contiguous(), top_k, norm_topk_prob)
 
 
-# Measured on an MI355X with OLMoE's shapes (bench.py --sweep): the weight-stream kernel
-# handles 16 rows of an expert per pass and wins while experts have about that many rows;
-# beyond that the MFMA tile kernel does. There is no third regime on this hardware.
+# Measured on an MI355X with OLMoE's shapes (bench.py --sweep): the weight-stream kernel wins
+# while the busiest expert has at most 16 rows (64 tokens: 0.244 vs 0.269 ms per layer; 96
+# tokens, 20 rows: 0.311 vs 0.260 ms), the MFMA tile kernel beyond. The reference's third
+# regime (a library GEMM per expert above 48 rows) does not exist on this hardware.
 GEMV_MAX_ROWS = 16
 GEMM_MAX_ROWS = 1 << 30
 
@@ -55,11 +58,13 @@ def pick(max_rows):
 
 def _auto(n_tokens, n_choices, n_experts):
     """Mode for "auto" without a device read. No expert can have more rows than there are
-    tokens, so up to GEMV_MAX_ROWS tokens the answer is certain; above that the mean rows
-    per expert stands in for the maximum (both kernels are correct for any routing)."""
+    tokens, so up to GEMV_MAX_ROWS tokens the answer is certain; above that the busiest expert
+    is estimated from the mean rows per expert (under near-uniform routing it sits about two
+    square roots of the mean above it). Both kernels are correct for any routing."""
     if n_tokens <= GEMV_MAX_ROWS:
         return "gemv"
-    return pick(-(-n_choices // n_experts))
+    mean = n_choices / n_experts
+    return pick(math.ceil(mean + 2.0 * math.sqrt(mean)))
 
 
 def ffn(x, a_rows, offsets, counts, wsorted, gate_up, down, rows, mode, host_counts=None):
