@@ -1,11 +1,13 @@
 // grouped_gemm: the prefill path. Every expert's slice of the sorted rows goes through that
 // expert's weights on fp16 MFMA tiles, all experts in one launch.
 //
-// Tile: 64*MI rows x 256 weight rows (MI = 1 or 2), K in slices of 64, 4 wavefronts (2 x 2), each
-// computing 32*MI rows x 128 weight rows as MI x 4 v_mfma_f32_32x32x16_f16 blocks with fp32 accumulators.
-// With SwiGLU the 256 weight rows are 128 gate rows and the 128 up rows of the same output
-// columns, and a wavefront holds gate and up of the same 64 columns, so the activation is
-// applied in registers. Weights are the MFMA M operand and rows the N operand: a lane ends
+// Tile: 64*MI rows x 256 weight rows (MI = 1 or 2), K in slices of 64, 4 wavefronts, each computing
+// all of the tile's rows x 64 weight rows as (2*MI) x 2 v_mfma_f32_32x32x16_f16 blocks with fp32
+// accumulators. With SwiGLU the 256 weight rows are 128 gate rows and the 128 up rows of the
+// same output columns, and a wavefront holds gate and up of the same 32 columns, so the
+// activation is applied in registers. Every wavefront sees every row of the tile, so 32-row
+// blocks past the end of the expert are skipped by all four: a ragged last tile costs what its
+// live blocks cost. Weights are the MFMA M operand and rows the N operand: a lane ends
 // up with runs of 4 consecutive output columns of one row and stores them as 8 bytes.
 //
 // Rows are gathered from the unsorted input inside the kernel (a_rows). A K-slice is 64 wide
@@ -24,6 +26,8 @@
 //
 // Replaces grouped_gemm_kernel / grouped_gemm of the reference
 // (switchyard/csrc/moe_kernels.cu:159-298); epilogue rounding points as :253-259.
+#include <type_traits>
+
 #include "common.h"
 
 namespace {
@@ -136,57 +140,68 @@ gemm_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const 
     for (int q = 0; q < NB; ++q) *reinterpret_cast<half8_t*>(bs + (lrow + 32 * q) * LDS_LD + lch) = rb[q];
   };
 
-  // ---- wavefront tile
-  const int wm = wave >> 1, wn = wave & 1;
+  // ---- wavefront tile: all of the tile's rows x 64 weight rows (wavefront w owns weight rows
+  // brow[0], brow[1]); row blocks past the expert's end are skipped, so a tile costs what its
+  // 32-row blocks cost and not what a full tile costs
   const int l32 = lane & 31, lk = (lane >> 5) * 8;
-  int brow[4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) brow[j] = SWIGLU ? (j >> 1) * COLS + wn * 64 + (j & 1) * 32 : wn * 128 + j * 32;
+  constexpr int RB = BM / 32;  // 32-row blocks per tile
+  int brow[2];
+  brow[0] = SWIGLU ? wave * 32 : wave * 64;
+  brow[1] = SWIGLU ? COLS + wave * 32 : wave * 64 + 32;
 
-  float16_t acc[MI][4];
+  float16_t acc[RB][2];
 #pragma unroll
-  for (int i = 0; i < MI; ++i)
+  for (int i = 0; i < RB; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  fetch(0);
   const int nk = (K + BK - 1) / BK;
-  const half_t* as = lds + (wm * 32 * MI + l32) * LDS_LD + lk;
+  const half_t* as = lds + l32 * LDS_LD + lk;
   const half_t* bs = lds + (BM + l32) * LDS_LD + lk;
-  for (int kt = 0; kt < nk; ++kt) {
-    if (kt) __syncthreads();  // every wavefront is done reading the previous slice
-    stash();
-    __syncthreads();
-    if (kt + 1 < nk) fetch((kt + 1) * BK);
+  // the K loop for LIVE live row blocks (a compile-time count: the loop body stays branch-free)
+  auto k_loop = [&](auto live_blocks) {
+    constexpr int LIVE = decltype(live_blocks)::value;
+    fetch(0);
+    for (int kt = 0; kt < nk; ++kt) {
+      if (kt) __syncthreads();  // every wavefront is done reading the previous slice
+      stash();
+      if (kt + 1 < nk) fetch((kt + 1) * BK);  // in flight during this slice's MFMAs
+      __syncthreads();
 #pragma unroll
-    for (int kk = 0; kk < BK; kk += 16) {
-      half8_t xf[MI], wf[4];
+      for (int kk = 0; kk < BK; kk += 16) {
+        half8_t xf[LIVE], wf[2];
 #pragma unroll
-      for (int i = 0; i < MI; ++i) xf[i] = *reinterpret_cast<const half8_t*>(as + i * 32 * LDS_LD + kk);
+        for (int i = 0; i < LIVE; ++i) xf[i] = *reinterpret_cast<const half8_t*>(as + i * 32 * LDS_LD + kk);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) wf[j] = *reinterpret_cast<const half8_t*>(bs + brow[j] * LDS_LD + kk);
+        for (int j = 0; j < 2; ++j) wf[j] = *reinterpret_cast<const half8_t*>(bs + brow[j] * LDS_LD + kk);
 #pragma unroll
-      for (int i = 0; i < MI; ++i)
+        for (int i = 0; i < LIVE; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[j], xf[i], acc[i][j], 0, 0, 0);
+          for (int j = 0; j < 2; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[j], xf[i], acc[i][j], 0, 0, 0);
+      }
     }
-  }
+  };
+  const int live = (nrows + 31) / 32;
+  if (RB == 4 && live == 4) k_loop(std::integral_constant<int, RB>{});
+  else if (RB == 4 && live == 3) k_loop(std::integral_constant<int, (RB > 3 ? 3 : RB)>{});
+  else if (live >= 2) k_loop(std::integral_constant<int, 2>{});
+  else k_loop(std::integral_constant<int, 1>{});
 
   // ---- epilogue: acc element 4*q + r of block (i, j) is row i*32 + l32, column 8*q + 4*(lane/32) + r
   const int chalf = (lane >> 5) * 4;
 #pragma unroll
-  for (int i = 0; i < MI; ++i) {
-    const int row = row0 + wm * 32 * MI + i * 32 + l32;
+  for (int i = 0; i < RB; ++i) {
+    const int row = row0 + i * 32 + l32;
     if (row >= row_end) continue;
     const float sc_row = SCALE ? (float)scale[row] : 1.f;
     half_t* crow = C + (size_t)row * Nout;
-    constexpr int NJ = SWIGLU ? 2 : 4;
+    constexpr int NJ = SWIGLU ? 1 : 2;
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
-      const int cbase = n0 + (SWIGLU ? wn * 64 + j * 32 : wn * 128 + j * 32) + chalf;
+      const int cbase = n0 + (SWIGLU ? wave * 32 : wave * 64 + j * 32) + chalf;
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int c0 = cbase + 8 * q;
@@ -194,7 +209,7 @@ gemm_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const 
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const float v = acc[i][j][4 * q + r];
-          if (SWIGLU) o[r] = swiglu_f16(v, acc[i][j + 2][4 * q + r]);
+          if (SWIGLU) o[r] = swiglu_f16(v, acc[i][1][4 * q + r]);
           else if (SCALE) o[r] = (half_t)((float)(half_t)v * sc_row);
           else o[r] = (half_t)v;
         }
