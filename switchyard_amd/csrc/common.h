@@ -68,6 +68,17 @@ __device__ __forceinline__ float wave_sum(float v) {
   return wave_allreduce(v, [](float a, float b) { return a + b; });
 }
 
+// SwiGLU with the reference's rounding points: gate and up are rounded to fp16, silu(gate) is
+// rounded to fp16, and so is the product (F.silu(gate) * up on fp16 tensors). The sigmoid uses
+// the hardware's exp2 and reciprocal (about 1 ulp each in fp32, far below the fp16 rounding);
+// exp2 overflows to +inf for very negative gates and the result is then -0, the right limit.
+__device__ __forceinline__ half_t swiglu_f16(float gate, float up) {
+  const float g = (float)(half_t)gate, u = (float)(half_t)up;
+  const float sig = __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(g * -1.4426950408889634f));
+  const float s = (float)(half_t)(g * sig);
+  return (half_t)(s * u);
+}
+
 __device__ __forceinline__ uint64_t lanemask_lt() {
   return (1ull << (threadIdx.x & 63)) - 1ull;
 }

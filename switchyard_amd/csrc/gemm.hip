@@ -17,15 +17,13 @@
 // computes meanwhile. LDS rows are padded to 144 bytes so that the 128-bit operand reads of
 // 16 consecutive lanes fall in distinct banks.
 //
-// The row tiles of all experts are laid end to end. The map from a tile to (expert, first
-// row) is rebuilt by every workgroup from `offsets` with one wavefront scan, so the host
-// needs neither the reference's tile_offsets tensor nor a device-to-host read; the grid is
-// sized for the worst case and surplus workgroups leave at once. Workgroups are renumbered
-// so that consecutive tiles, which share rows or weights, run on the same XCD and meet in
-// its L2.
+// The map from a workgroup to its tile is rebuilt on the device from `offsets` (find_tile), so
+// the host needs neither the reference's tile_offsets tensor nor a device-to-host read.
 //
 // Replaces grouped_gemm_kernel / grouped_gemm of the reference
 // (switchyard/csrc/moe_kernels.cu:159-298); epilogue rounding points as :253-259.
+#include <stdlib.h>
+
 #include <type_traits>
 
 #include "common.h"
@@ -38,53 +36,88 @@ constexpr int LDS_LD = BK + 8;   // halves per LDS row (144 bytes)
 constexpr int GEMM_THREADS = 256;
 constexpr int XCDS = 8;
 
-__device__ __forceinline__ half_t swiglu_f16(float gate, float up) {
-  const float g = (float)(half_t)gate, u = (float)(half_t)up;
-  const float s = (float)(half_t)(g / (1.f + expf(-g)));
-  return (half_t)(s * u);
+// Inclusive prefix sum over the lanes of a wavefront.
+__device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
+  for (int o = 1; o < WAVE; o <<= 1) {
+    const int up = __shfl_up(v, o, WAVE);
+    if (lane >= o) v += up;
+  }
+  return v;
+}
+
+// Which tile this workgroup computes. The row tiles of all experts form two lists, the full
+// tiles of BM rows, expert by expert, and the ragged last tiles; each row tile is followed by
+// its column tiles. Each list is cut into 8 equal runs, one per XCD (workgroups are dealt
+// round-robin to the XCDs), so that neighbours, which share rows or weights, meet in one L2 and
+// every XCD gets the same share of both kinds whatever the routing; an XCD works through its
+// full tiles first, so the cheap tiles fill the end of the launch. The first wavefront
+// rebuilds the lists from `offsets` with two scans; the grid is sized for the worst case and
+// surplus workgroups leave at once.
+// Returns false for a surplus workgroup; must be called by every thread of the workgroup.
+template <int BM>
+__device__ __forceinline__ bool find_tile(const int* __restrict__ offsets, int E, int ncol_tiles, int* s_tile,
+                                          int& e, int& row0, int& row_end, int& col_tile) {
+  const int tid = threadIdx.x, lane = tid & 63;
+  if (tid == 0) s_tile[0] = -1;
+  __syncthreads();
+  if (tid < WAVE) {
+    int full_total = 0, ragged_total = 0;
+    for (int e0 = 0; e0 < E; e0 += WAVE) {
+      const int x = e0 + lane;
+      const int n = x < E ? offsets[x + 1] - offsets[x] : 0;
+      full_total += n / BM;
+      ragged_total += (n % BM) != 0;
+    }
+    full_total = wave_inclusive_scan(full_total, lane);
+    ragged_total = wave_inclusive_scan(ragged_total, lane);
+    full_total = __shfl(full_total, WAVE - 1, WAVE);
+    ragged_total = __shfl(ragged_total, WAVE - 1, WAVE);
+    const long full_tiles = (long)full_total * ncol_tiles, ragged_tiles = (long)ragged_total * ncol_tiles;
+    const long full_per_xcd = (full_tiles + XCDS - 1) / XCDS, ragged_per_xcd = (ragged_tiles + XCDS - 1) / XCDS;
+    const long slot = blockIdx.x / XCDS, xcd = blockIdx.x % XCDS;
+    const bool ragged = slot >= full_per_xcd;
+    const long logical = ragged ? xcd * ragged_per_xcd + slot - full_per_xcd : xcd * full_per_xcd + slot;
+    if (logical < (ragged ? ragged_tiles : full_tiles) && slot < full_per_xcd + ragged_per_xcd) {
+      const int want = (int)(logical / ncol_tiles);
+      int run = 0;
+      for (int e0 = 0; e0 < E; e0 += WAVE) {
+        const int x = e0 + lane;
+        const int first = x < E ? offsets[x] : 0, last = x < E ? offsets[x + 1] : 0;
+        const int full = (last - first) / BM;
+        const int mine = ragged ? ((last - first) % BM != 0) : full;
+        const int inc = wave_inclusive_scan(mine, lane);
+        const int lo = run + inc - mine;
+        if (want >= lo && want < lo + mine) {
+          s_tile[0] = x;
+          s_tile[1] = first + (ragged ? full : want - lo) * BM;
+          s_tile[2] = last;
+          s_tile[3] = (int)(logical % ncol_tiles);
+        }
+        run += __shfl(inc, WAVE - 1, WAVE);
+      }
+    }
+  }
+  __syncthreads();
+  e = __builtin_amdgcn_readfirstlane(s_tile[0]);
+  if (e < 0) return false;
+  row0 = __builtin_amdgcn_readfirstlane(s_tile[1]);
+  row_end = __builtin_amdgcn_readfirstlane(s_tile[2]);
+  col_tile = __builtin_amdgcn_readfirstlane(s_tile[3]);
+  return true;
 }
 
 template <int MI, bool SWIGLU, bool SCALE>
 __global__ void __launch_bounds__(GEMM_THREADS, 2)
 gemm_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const half_t* __restrict__ B,
             const int* __restrict__ offsets, int E, int Nout, int K, const half_t* __restrict__ scale,
-            half_t* __restrict__ C, int ncol_tiles, int per_xcd) {
+            half_t* __restrict__ C, int ncol_tiles) {
   constexpr int BM = 64 * MI;  // rows per tile
   __shared__ __attribute__((aligned(16))) half_t lds[(BM + BW) * LDS_LD];
-  __shared__ int s_tile[3];
+  __shared__ int s_tile[4];
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-
-  // consecutive logical tiles on one XCD (workgroups are dealt round-robin to the XCDs)
-  const int logical = (blockIdx.x % XCDS) * per_xcd + blockIdx.x / XCDS;
-  const int row_tile = logical / ncol_tiles, col_tile = logical % ncol_tiles;
-
-  if (tid == 0) s_tile[0] = -1;
-  __syncthreads();
-  if (wave == 0) {
-    int run = 0;
-    for (int e0 = 0; e0 < E; e0 += WAVE) {
-      const int e = e0 + lane;
-      const int first = e < E ? offsets[e] : 0, last = e < E ? offsets[e + 1] : 0;
-      const int tiles = (last - first + BM - 1) / BM;
-      int inc = tiles;
-      for (int o = 1; o < WAVE; o <<= 1) {
-        const int up = __shfl_up(inc, o, WAVE);
-        if (lane >= o) inc += up;
-      }
-      const int lo = run + inc - tiles;
-      if (row_tile >= lo && row_tile < lo + tiles) {
-        s_tile[0] = e;
-        s_tile[1] = first + (row_tile - lo) * BM;
-        s_tile[2] = last;
-      }
-      run += __shfl(inc, WAVE - 1, WAVE);
-    }
-  }
-  __syncthreads();
-  const int e = s_tile[0];
-  if (e < 0) return;
-  const int row0 = s_tile[1], row_end = s_tile[2];
+  int e, row0, row_end, col_tile;
+  if (!find_tile<BM>(offsets, E, ncol_tiles, s_tile, e, row0, row_end, col_tile)) return;
   const int nrows = min(BM, row_end - row0);
 
   constexpr int COLS = SWIGLU ? BW / 2 : BW;  // output columns per tile
@@ -225,6 +258,286 @@ gemm_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const 
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// The tile for many rows per expert: 256 rows x 256 weight rows, 8 wavefronts (2 x 4, each 128
+// rows x 64 weight rows), one workgroup per CU.
+//
+// A 128-row tile asks the CU for 48 KB of operands per 1024 MFMA cycles, more than the path
+// from L2 delivers (about 44 B per clock per CU for rows of 128 bytes, half of that for rows
+// of 64), and moving them through registers into LDS costs more LDS write cycles than the
+// MFMAs take. This tile halves the bytes per flop and lets the memory pipeline write LDS
+// itself (buffer loads with the LDS modifier): no staging registers and no ds_write.
+//
+// All 160 KB of LDS are operand slices of 32 KB: two of the rows, three of the weight rows.
+// The rows of a tile are shared by all its column tiles and mostly hit in L2; the weights are
+// read from HBM by the first of the few row tiles that share them, and such a load is away for
+// longer than the MFMAs of a slice take, so weights are fetched two slices ahead and rows one.
+// A slice is four K-steps; the one barrier per slice sits before the last step, where that
+// step's operands are already in registers: it publishes slice i + 1 and says that every
+// wavefront has read all of slice i, so the MFMAs of the last step run while the first
+// operands of slice i + 1 are read and the loads of rows i + 2 and weights i + 3 go out, one
+// at a time between the MFMAs, into the buffers that slice i has just left.
+//
+// One such load writes the 64 lanes' 16 bytes to 1 KB of consecutive LDS: 8 unpadded rows of
+// 128 bytes. Which 16 bytes of its row a lane fetches is therefore chosen so that the operand
+// reads stay free of bank conflicts: chunk c of row r sits at position c ^ ((r >> 1) & 7).
+// The compiler is not told about these loads (it would wait for all of them before every LDS
+// read), so the waits are written by hand.
+constexpr int BIG_BM = 256, BIG_THREADS = 512;
+constexpr int BIG_BK = 64;                                        // K per slice
+constexpr int BIG_STEPS = BIG_BK / 16;                            // MFMA K-steps per slice
+constexpr int BIG_ROW_BYTES = BIG_BK * 2;                         // 128
+constexpr int BIG_A_BYTES = BIG_BM * BIG_ROW_BYTES;               // 32 KB: a slice of the rows
+constexpr int BIG_B_BYTES = BW * BIG_ROW_BYTES;                   // 32 KB: a slice of the weight rows
+constexpr int BIG_A_STAGES = 2, BIG_B_STAGES = 3;                 // all 160 KB of LDS
+constexpr int BIG_LOADS = BIG_A_BYTES / (BIG_THREADS * 16);       // 4 per thread, slice and operand
+
+typedef int int4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ int4_t buffer_descriptor(const void* base, unsigned bytes) {
+  const uint64_t a = (uint64_t)base;
+  int4_t d;
+  d[0] = __builtin_amdgcn_readfirstlane((int)(unsigned)a);
+  d[1] = __builtin_amdgcn_readfirstlane((int)((unsigned)(a >> 32) & 0xffffu));
+  d[2] = __builtin_amdgcn_readfirstlane((int)bytes);
+  d[3] = 0x00020000;
+  return d;
+}
+
+// 16 bytes per lane from buffer offset voffset + soffset to LDS address lds_addr + 16 * lane.
+// Only voffset is checked against the size of the buffer.
+__device__ __forceinline__ void load_to_lds(int4_t rsrc, unsigned voffset, unsigned soffset, unsigned lds_addr) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "buffer_load_dwordx4 %1, %2, %3 offen lds"
+      :
+      : "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset)
+      : "memory");  // m0 is not otherwise used in this file: the compiler needs it for no LDS or lane instruction here
+}
+
+template <bool SWIGLU, bool SCALE>
+__global__ void __launch_bounds__(BIG_THREADS, 1)
+gemm_big_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const half_t* __restrict__ B,
+                const int* __restrict__ offsets, int E, int Nout, int K, const half_t* __restrict__ scale,
+                half_t* __restrict__ C, int ncol_tiles) {
+  constexpr int BM = BIG_BM;
+  __shared__ __attribute__((aligned(1024))) char lds[BIG_A_STAGES * BIG_A_BYTES + BIG_B_STAGES * BIG_B_BYTES];
+  static_assert(sizeof(lds) == 160 * 1024, "the whole LDS of a CU");
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  int e, row0, row_end, col_tile;
+  // the tile lookup borrows the first bytes of the operand buffers
+  if (!find_tile<BM>(offsets, E, ncol_tiles, reinterpret_cast<int*>(lds), e, row0, row_end, col_tile)) return;
+  __syncthreads();  // everyone has read the lookup's result before loads overwrite it
+  const int nrows = min(BM, row_end - row0);
+
+  constexpr int COLS = SWIGLU ? BW / 2 : BW;
+  const int n0 = col_tile * COLS;
+  const int Nfull = SWIGLU ? 2 * Nout : Nout;
+  const half_t* Be = B + (size_t)e * Nfull * K;
+
+  // ---- loader: load q of wavefront w fills LDS rows 8 * (8 * q + w) .. + 8, of the tile's rows
+  // and of its weight rows; lane l brings row l / 8 of them, and of that row the chunk that
+  // belongs at position l % 8
+  constexpr unsigned OUT_OF_RANGE = 0x80000000u;
+  const int4_t arsrc = buffer_descriptor(A, 0x7fffffffu);
+  const int4_t brsrc = buffer_descriptor(Be, (unsigned)((size_t)Nfull * K * 2));
+  unsigned oa[4], ob[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int r = 8 * (8 * q + wave) + (lane >> 3);
+    const unsigned chunk = (unsigned)((lane & 7) ^ ((r >> 1) & 7));
+    const int src = r < nrows ? (a_rows ? a_rows[row0 + r] : row0 + r) : 0;
+    oa[q] = r < nrows ? ((unsigned)src * (unsigned)K + chunk * 8u) * 2u : OUT_OF_RANGE;
+    int wr, col;
+    if (SWIGLU) {
+      col = n0 + (r & (COLS - 1));
+      wr = r < COLS ? col : Nout + col;
+    } else {
+      col = n0 + r;
+      wr = col;
+    }
+    ob[q] = col < Nout ? ((unsigned)wr * (unsigned)K + chunk * 8u) * 2u : OUT_OF_RANGE;
+  }
+  const int nk = K / BIG_BK;
+  const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) char*)lds;
+  const unsigned wave_base = __builtin_amdgcn_readfirstlane(lds_base + wave * 1024);
+  // load q (0 .. 3) of the rows, or of the weight rows, of slice kt into buffer `stage`; past K
+  // it is still issued, out of range (only the per-lane offset is checked), and moves nothing
+  auto issue_rows = [&](int kt, int stage, int q) {
+    load_to_lds(arsrc, kt < nk ? oa[q] : OUT_OF_RANGE, (unsigned)kt * (BIG_BK * 2), wave_base + stage * BIG_A_BYTES + q * 8192);
+  };
+  auto issue_weights = [&](int kt, int stage, int q) {
+    load_to_lds(brsrc, kt < nk ? ob[q] : OUT_OF_RANGE, (unsigned)kt * (BIG_BK * 2),
+                wave_base + BIG_A_STAGES * BIG_A_BYTES + stage * BIG_B_BYTES + q * 8192);
+  };
+  static_assert(BIG_LOADS == 4, "oa and ob hold four loads per wavefront, slice and operand");
+
+  // ---- wavefront tile: rows wm * 128 .. + 128, weight rows brow[0] .. + 32 and brow[1] .. + 32
+  const int wm = wave >> 2, wn = wave & 3;
+  const int l32 = lane & 31;
+  int brow[2];
+  brow[0] = SWIGLU ? wn * 32 : wn * 64;
+  brow[1] = SWIGLU ? COLS + wn * 32 : wn * 64 + 32;
+  // byte offset inside a row of K-step s (16 halves = chunks 2s and 2s + 1; the upper 32 lanes
+  // take the second); every 32-row block starts at a multiple of 32, so the swizzle depends on
+  // the lane alone
+  int koff[BIG_STEPS];
+#pragma unroll
+  for (int s = 0; s < BIG_STEPS; ++s) koff[s] = (((2 * s + (lane >> 5)) ^ ((l32 >> 1) & 7)) * 16);
+
+  float16_t acc[4][2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  const char* as = lds + (wm * 128 + l32) * BIG_ROW_BYTES;
+  const char* bs = lds + BIG_A_STAGES * BIG_A_BYTES + l32 * BIG_ROW_BYTES;
+
+  // The K loop for LIVE live row blocks (a compile-time count: the loop body is branch-free).
+  auto k_loop = [&](auto live_blocks) {
+    constexpr int LIVE = decltype(live_blocks)::value;
+    constexpr int READS = LIVE > 0 ? LIVE + 2 : 0, MFMAS = 2 * LIVE;
+    constexpr int PAIRS = READS < MFMAS ? READS : MFMAS;
+    half8_t xf[2][LIVE > 0 ? LIVE : 1], wf[2][2];  // operands of even and odd K-steps
+    // operand r of K-step s of the slice whose rows start at byte sa and weights at sb: the two
+    // weight blocks, then the row blocks
+    auto read = [&](int sa, int sb, int s, int r) {
+      if (r < 2) wf[s & 1][r] = *reinterpret_cast<const half8_t*>(bs + sb + brow[r] * BIG_ROW_BYTES + koff[s]);
+      else xf[s & 1][r - 2] = *reinterpret_cast<const half8_t*>(as + sa + (r - 2) * 32 * BIG_ROW_BYTES + koff[s]);
+    };
+    auto mfma = [&](int s, int m) {
+      const int i = m >> 1, j = m & 1;
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[s & 1][j], xf[s & 1][i], acc[i][j], 0, 0, 0);
+    };
+    // issue order: rows 0, weights 0 | rows 1, weights 1 | weights 2; from then on rows i + 2
+    // and then weights i + 3, so that "slice i + 1 has landed" is always "all but the last 4"
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+#pragma unroll
+      for (int q = 0; q < BIG_LOADS; ++q) issue_rows(p, p, q);
+#pragma unroll
+      for (int q = 0; q < BIG_LOADS; ++q) issue_weights(p, p, q);
+    }
+#pragma unroll
+    for (int q = 0; q < BIG_LOADS; ++q) issue_weights(2, 2, q);
+    asm volatile("s_waitcnt vmcnt(12)" ::: "memory");  // slice 0 has landed
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < READS; ++r) read(0, 0, 0, r);
+    int a_stage = 0, b_stage = 0;  // where slice kt is
+    for (int kt = 0; kt < nk; ++kt) {
+      const int a_next = a_stage ^ 1, b_next = b_stage == BIG_B_STAGES - 1 ? 0 : b_stage + 1;
+      const int sa = a_stage * BIG_A_BYTES, sb = b_stage * BIG_B_BYTES;
+      // all steps but the last, each with the reads of the next step behind its MFMAs
+#pragma unroll
+      for (int s = 0; s < BIG_STEPS - 1; ++s) {
+#pragma unroll
+        for (int r = 0; r < READS; ++r) read(sa, sb, s + 1, r);
+#pragma unroll
+        for (int m = 0; m < MFMAS; ++m) mfma(s, m);
+      }
+#pragma unroll
+      for (int s = 0; s < BIG_STEPS - 1; ++s) {
+#pragma unroll
+        for (int n = 0; n < PAIRS; ++n) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        if (READS > PAIRS) __builtin_amdgcn_sched_group_barrier(0x100, READS - PAIRS, 0);
+        if (MFMAS > PAIRS) __builtin_amdgcn_sched_group_barrier(0x008, MFMAS - PAIRS, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      // slice kt + 1 has landed (the weights of slice kt + 2 may be out) and this wavefront's
+      // reads of slice kt are complete
+      asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
+      static_assert(BIG_LOADS == 4, "the count in the wait above");
+      __syncthreads();
+      // the last step in eight parts, each followed by one load: rows kt + 2, then weights kt + 3
+#pragma unroll
+      for (int part = 0; part < 2 * BIG_LOADS; ++part) {
+#pragma unroll
+        for (int r = 0; r < READS; ++r)
+          if (r * 2 * BIG_LOADS / (READS > 0 ? READS : 1) == part) read(a_next * BIG_A_BYTES, b_next * BIG_B_BYTES, 0, r);
+#pragma unroll
+        for (int m = 0; m < MFMAS; ++m)
+          if (m * 2 * BIG_LOADS / (MFMAS > 0 ? MFMAS : 1) == part) mfma(BIG_STEPS - 1, m);
+        __builtin_amdgcn_sched_barrier(0);
+        if (part < BIG_LOADS) issue_rows(kt + 2, a_stage, part);
+        else issue_weights(kt + 3, b_stage, part - BIG_LOADS);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      a_stage = a_next;
+      b_stage = b_next;
+    }
+  };
+  const int live = max(0, min(4, (nrows - wm * 128 + 31) / 32));
+  switch (live) {
+    case 4: k_loop(std::integral_constant<int, 4>{}); break;
+    case 3: k_loop(std::integral_constant<int, 3>{}); break;
+    case 2: k_loop(std::integral_constant<int, 2>{}); break;
+    case 1: k_loop(std::integral_constant<int, 1>{}); break;
+    default: k_loop(std::integral_constant<int, 0>{}); break;
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no load may land in LDS after this workgroup has given it back
+
+  // ---- epilogue: acc element 4*q + r of block (i, j) is row i*32 + l32, column 8*q + 4*(lane/32) + r
+  const int chalf = (lane >> 5) * 4;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = row0 + wm * 128 + i * 32 + l32;
+    if (row >= row_end) continue;
+    const float sc_row = SCALE ? (float)scale[row] : 1.f;
+    half_t* crow = C + (size_t)row * Nout;
+    constexpr int NJ = SWIGLU ? 1 : 2;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const int cbase = n0 + (SWIGLU ? wn * 32 : wn * 64 + j * 32) + chalf;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int c0 = cbase + 8 * q;
+        half4_t o;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float v = acc[i][j][4 * q + r];
+          if (SWIGLU) o[r] = swiglu_f16(v, acc[i][1][4 * q + r]);
+          else if (SCALE) o[r] = (half_t)((float)(half_t)v * sc_row);
+          else o[r] = (half_t)v;
+        }
+        if (c0 + 3 < Nout && (Nout & 3) == 0) {
+          *reinterpret_cast<half4_t*>(crow + c0) = o;
+        } else {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (c0 + r < Nout) crow[c0 + r] = o[r];
+        }
+      }
+    }
+  }
+}
+
+int launch_gemm_big(const half_t* a, const int32_t* a_rows, const half_t* b, const int32_t* offsets, int E, int rows,
+                    int Nout, int K, int swiglu, const half_t* s, half_t* c, hipStream_t st) {
+  const int cols = swiglu ? BW / 2 : BW;
+  const int ncol_tiles = (Nout + cols - 1) / cols;
+  const long max_row_tiles = rows / BIG_BM + (E < rows ? E : rows);
+  const long total = max_row_tiles * ncol_tiles;
+  if (total >= (1l << 31) - XCDS) return sy_fail(SY_ERR_ARG, "grouped_gemm: too many tiles");
+  const int per_xcd = (int)((total + XCDS - 1) / XCDS) + 1;  // full and ragged tiles are each rounded up to 8
+  const int grid = per_xcd * XCDS;
+  if (swiglu)
+    gemm_big_kernel<true, false><<<grid, BIG_THREADS, 0, st>>>(a, a_rows, b, offsets, E, Nout, K, nullptr, c, ncol_tiles);
+  else if (s)
+    gemm_big_kernel<false, true><<<grid, BIG_THREADS, 0, st>>>(a, a_rows, b, offsets, E, Nout, K, s, c, ncol_tiles);
+  else
+    gemm_big_kernel<false, false><<<grid, BIG_THREADS, 0, st>>>(a, a_rows, b, offsets, E, Nout, K, nullptr, c, ncol_tiles);
+  return sy_check_launch("grouped_gemm");
+}
+
 template <int MI>
 int launch_gemm(const half_t* a, const int32_t* a_rows, const half_t* b, const int32_t* offsets, int E, int rows,
                 int Nout, int K, int swiglu, const half_t* s, half_t* c, hipStream_t st) {
@@ -235,14 +548,14 @@ int launch_gemm(const half_t* a, const int32_t* a_rows, const half_t* b, const i
   const long max_row_tiles = rows / BM + (E < rows ? E : rows);
   const long total = max_row_tiles * ncol_tiles;
   if (total >= (1l << 31) - XCDS) return sy_fail(SY_ERR_ARG, "grouped_gemm: too many tiles");
-  const int per_xcd = (int)((total + XCDS - 1) / XCDS);
+  const int per_xcd = (int)((total + XCDS - 1) / XCDS) + 1;  // full and ragged tiles are each rounded up to 8
   const int grid = per_xcd * XCDS;
   if (swiglu)
-    gemm_kernel<MI, true, false><<<grid, GEMM_THREADS, 0, st>>>(a, a_rows, b, offsets, E, Nout, K, nullptr, c, ncol_tiles, per_xcd);
+    gemm_kernel<MI, true, false><<<grid, GEMM_THREADS, 0, st>>>(a, a_rows, b, offsets, E, Nout, K, nullptr, c, ncol_tiles);
   else if (s)
-    gemm_kernel<MI, false, true><<<grid, GEMM_THREADS, 0, st>>>(a, a_rows, b, offsets, E, Nout, K, s, c, ncol_tiles, per_xcd);
+    gemm_kernel<MI, false, true><<<grid, GEMM_THREADS, 0, st>>>(a, a_rows, b, offsets, E, Nout, K, s, c, ncol_tiles);
   else
-    gemm_kernel<MI, false, false><<<grid, GEMM_THREADS, 0, st>>>(a, a_rows, b, offsets, E, Nout, K, nullptr, c, ncol_tiles, per_xcd);
+    gemm_kernel<MI, false, false><<<grid, GEMM_THREADS, 0, st>>>(a, a_rows, b, offsets, E, Nout, K, nullptr, c, ncol_tiles);
   return sy_check_launch("grouped_gemm");
 }
 
@@ -266,6 +579,10 @@ extern "C" SY_API int sy_grouped_gemm(const void* A, const int32_t* a_rows, cons
   const half_t* b = (const half_t*)B;
   const half_t* s = (const half_t*)scale;
   half_t* c = (half_t*)C;
-  if (typical <= 64) return launch_gemm<1>(a, a_rows, b, offsets, E, rows, Nout, K, swiglu, s, c, (hipStream_t)stream);
+  static const int forced = getenv("SY_GEMM_TILE") ? atoi(getenv("SY_GEMM_TILE")) : 0;
+  const int tile = forced ? forced : typical <= 64 ? 64 : typical <= 192 ? 128 : 256;  // 256 needs K % 64 == 0, else 128
+  if (tile == 256 && K % BIG_BK == 0)
+    return launch_gemm_big(a, a_rows, b, offsets, E, rows, Nout, K, swiglu, s, c, (hipStream_t)stream);
+  if (tile == 64) return launch_gemm<1>(a, a_rows, b, offsets, E, rows, Nout, K, swiglu, s, c, (hipStream_t)stream);
   return launch_gemm<2>(a, a_rows, b, offsets, E, rows, Nout, K, swiglu, s, c, (hipStream_t)stream);
 }

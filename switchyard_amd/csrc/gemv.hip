@@ -51,13 +51,6 @@ __device__ __forceinline__ half8_t load_stream(__amdgpu_buffer_rsrc_t rsrc, unsi
 }
 constexpr unsigned OUT_OF_RANGE = 0x80000000u;
 
-__device__ __forceinline__ half_t swiglu_f16(float gate, float up) {
-  // the rounding points of the fp16 torch graph: gate and up to f16, silu in fp32 to f16, product to f16
-  const float g = (float)(half_t)gate, u = (float)(half_t)up;
-  const float s = (float)(half_t)(g / (1.f + expf(-g)));
-  return (half_t)(s * u);
-}
-
 __device__ __forceinline__ half4_t lo4(half8_t v) { return __builtin_shufflevector(v, v, 0, 1, 2, 3); }
 __device__ __forceinline__ half4_t hi4(half8_t v) { return __builtin_shufflevector(v, v, 4, 5, 6, 7); }
 
