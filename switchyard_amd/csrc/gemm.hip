@@ -22,8 +22,6 @@
 //
 // Replaces grouped_gemm_kernel / grouped_gemm of the reference
 // (switchyard/csrc/moe_kernels.cu:159-298); epilogue rounding points as :253-259.
-#include <stdlib.h>
-
 #include <type_traits>
 
 #include "common.h"
@@ -45,15 +43,18 @@ __device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
   return v;
 }
 
-// Which tile this workgroup computes. The row tiles of all experts form two lists, the full
-// tiles of BM rows, expert by expert, and the ragged last tiles; each row tile is followed by
-// its column tiles. Each list is cut into 8 equal runs, one per XCD (workgroups are dealt
-// round-robin to the XCDs), so that neighbours, which share rows or weights, meet in one L2 and
-// every XCD gets the same share of both kinds whatever the routing; an XCD works through its
-// full tiles first, so the cheap tiles fill the end of the launch. The first wavefront
-// rebuilds the lists from `offsets` with two scans; the grid is sized for the worst case and
-// surplus workgroups leave at once.
-// Returns false for a surplus workgroup; must be called by every thread of the workgroup.
+// Which tile this workgroup computes. An expert with n rows gets ceil(n / BM) row tiles of equal
+// height (a multiple of 32, the last one takes what is left): a short remainder tile would
+// stream the expert's weights again for a handful of rows, equal tiles all carry enough MFMA
+// work to cover their loads, and no 32-row block is computed that a BM-high tiling would not
+// compute. The row tiles of all experts are laid end to end, each followed by its column
+// tiles, and the list is cut into 8 equal runs, one per XCD (workgroups are dealt round-robin
+// to the XCDs), so that neighbours, which share rows or weights, meet in one L2 and every XCD
+// gets the same share whatever the routing. The first wavefront rebuilds the list from
+// `offsets` with two scans; the grid is sized for the worst case and surplus workgroups leave
+// at once.
+// Returns false for a surplus workgroup, else the expert, the tile's first row and the row
+// after its last; must be called by every thread of the workgroup.
 template <int BM>
 __device__ __forceinline__ bool find_tile(const int* __restrict__ offsets, int E, int ncol_tiles, int* s_tile,
                                           int& e, int& row0, int& row_end, int& col_tile) {
@@ -61,36 +62,32 @@ __device__ __forceinline__ bool find_tile(const int* __restrict__ offsets, int E
   if (tid == 0) s_tile[0] = -1;
   __syncthreads();
   if (tid < WAVE) {
-    int full_total = 0, ragged_total = 0;
+    int row_tiles = 0;
     for (int e0 = 0; e0 < E; e0 += WAVE) {
       const int x = e0 + lane;
       const int n = x < E ? offsets[x + 1] - offsets[x] : 0;
-      full_total += n / BM;
-      ragged_total += (n % BM) != 0;
+      row_tiles += (n + BM - 1) / BM;
     }
-    full_total = wave_inclusive_scan(full_total, lane);
-    ragged_total = wave_inclusive_scan(ragged_total, lane);
-    full_total = __shfl(full_total, WAVE - 1, WAVE);
-    ragged_total = __shfl(ragged_total, WAVE - 1, WAVE);
-    const long full_tiles = (long)full_total * ncol_tiles, ragged_tiles = (long)ragged_total * ncol_tiles;
-    const long full_per_xcd = (full_tiles + XCDS - 1) / XCDS, ragged_per_xcd = (ragged_tiles + XCDS - 1) / XCDS;
-    const long slot = blockIdx.x / XCDS, xcd = blockIdx.x % XCDS;
-    const bool ragged = slot >= full_per_xcd;
-    const long logical = ragged ? xcd * ragged_per_xcd + slot - full_per_xcd : xcd * full_per_xcd + slot;
-    if (logical < (ragged ? ragged_tiles : full_tiles) && slot < full_per_xcd + ragged_per_xcd) {
+    row_tiles = __shfl(wave_inclusive_scan(row_tiles, lane), WAVE - 1, WAVE);
+    const long total = (long)row_tiles * ncol_tiles;
+    const long per_xcd = (total + XCDS - 1) / XCDS;
+    const long slot = blockIdx.x / XCDS;
+    const long logical = (blockIdx.x % XCDS) * per_xcd + slot;
+    if (slot < per_xcd && logical < total) {
       const int want = (int)(logical / ncol_tiles);
       int run = 0;
       for (int e0 = 0; e0 < E; e0 += WAVE) {
         const int x = e0 + lane;
         const int first = x < E ? offsets[x] : 0, last = x < E ? offsets[x + 1] : 0;
-        const int full = (last - first) / BM;
-        const int mine = ragged ? ((last - first) % BM != 0) : full;
+        const int mine = (last - first + BM - 1) / BM;
         const int inc = wave_inclusive_scan(mine, lane);
         const int lo = run + inc - mine;
         if (want >= lo && want < lo + mine) {
+          const int height = ((last - first + mine - 1) / mine + 31) & ~31;
+          const int begin = first + (want - lo) * height;
           s_tile[0] = x;
-          s_tile[1] = first + (ragged ? full : want - lo) * BM;
-          s_tile[2] = last;
+          s_tile[1] = begin;
+          s_tile[2] = min(begin + height, last);
           s_tile[3] = (int)(logical % ncol_tiles);
         }
         run += __shfl(inc, WAVE - 1, WAVE);
@@ -283,14 +280,13 @@ gemm_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const 
 // reads stay free of bank conflicts: chunk c of row r sits at position c ^ ((r >> 1) & 7).
 // The compiler is not told about these loads (it would wait for all of them before every LDS
 // read), so the waits are written by hand.
-constexpr int BIG_BM = 256, BIG_THREADS = 512;
+constexpr int BIG_BM = 256;
 constexpr int BIG_BK = 64;                                        // K per slice
 constexpr int BIG_STEPS = BIG_BK / 16;                            // MFMA K-steps per slice
 constexpr int BIG_ROW_BYTES = BIG_BK * 2;                         // 128
 constexpr int BIG_A_BYTES = BIG_BM * BIG_ROW_BYTES;               // 32 KB: a slice of the rows
 constexpr int BIG_B_BYTES = BW * BIG_ROW_BYTES;                   // 32 KB: a slice of the weight rows
 constexpr int BIG_A_STAGES = 2, BIG_B_STAGES = 3;                 // all 160 KB of LDS
-constexpr int BIG_LOADS = BIG_A_BYTES / (BIG_THREADS * 16);       // 4 per thread, slice and operand
 
 typedef int int4_t __attribute__((ext_vector_type(4)));
 
@@ -316,12 +312,18 @@ __device__ __forceinline__ void load_to_lds(int4_t rsrc, unsigned voffset, unsig
       : "memory");  // m0 is not otherwise used in this file: the compiler needs it for no LDS or lane instruction here
 }
 
-template <bool SWIGLU, bool SCALE>
-__global__ void __launch_bounds__(BIG_THREADS, 1)
+// WN wavefronts side by side over the weight rows, two over the rows: 2 x 4 wavefronts of 128 rows x
+// 64 weight rows, or 2 x 2 of 128 x 128, which read a third less from LDS per MFMA and have a
+// SIMD each.
+template <int WN, bool SWIGLU, bool SCALE>
+__global__ void __launch_bounds__(2 * WN * WAVE, 1)
 gemm_big_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const half_t* __restrict__ B,
                 const int* __restrict__ offsets, int E, int Nout, int K, const half_t* __restrict__ scale,
                 half_t* __restrict__ C, int ncol_tiles) {
   constexpr int BM = BIG_BM;
+  constexpr int WAVES = 2 * WN, THREADS = WAVES * WAVE;
+  constexpr int NB = BW / (32 * WN);                    // 32-row weight blocks per wavefront
+  constexpr int LOADS = BIG_A_BYTES / (THREADS * 16);   // per thread, slice and operand
   __shared__ __attribute__((aligned(1024))) char lds[BIG_A_STAGES * BIG_A_BYTES + BIG_B_STAGES * BIG_B_BYTES];
   static_assert(sizeof(lds) == 160 * 1024, "the whole LDS of a CU");
 
@@ -337,16 +339,16 @@ gemm_big_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, co
   const int Nfull = SWIGLU ? 2 * Nout : Nout;
   const half_t* Be = B + (size_t)e * Nfull * K;
 
-  // ---- loader: load q of wavefront w fills LDS rows 8 * (8 * q + w) .. + 8, of the tile's rows
+  // ---- loader: load q of wavefront w fills LDS rows 8 * (WAVES * q + w) .. + 8, of the tile's rows
   // and of its weight rows; lane l brings row l / 8 of them, and of that row the chunk that
   // belongs at position l % 8
   constexpr unsigned OUT_OF_RANGE = 0x80000000u;
   const int4_t arsrc = buffer_descriptor(A, 0x7fffffffu);
   const int4_t brsrc = buffer_descriptor(Be, (unsigned)((size_t)Nfull * K * 2));
-  unsigned oa[4], ob[4];
+  unsigned oa[LOADS], ob[LOADS];
 #pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    const int r = 8 * (8 * q + wave) + (lane >> 3);
+  for (int q = 0; q < LOADS; ++q) {
+    const int r = 8 * (WAVES * q + wave) + (lane >> 3);
     const unsigned chunk = (unsigned)((lane & 7) ^ ((r >> 1) & 7));
     const int src = r < nrows ? (a_rows ? a_rows[row0 + r] : row0 + r) : 0;
     oa[q] = r < nrows ? ((unsigned)src * (unsigned)K + chunk * 8u) * 2u : OUT_OF_RANGE;
@@ -363,23 +365,26 @@ gemm_big_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, co
   const int nk = K / BIG_BK;
   const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) char*)lds;
   const unsigned wave_base = __builtin_amdgcn_readfirstlane(lds_base + wave * 1024);
-  // load q (0 .. 3) of the rows, or of the weight rows, of slice kt into buffer `stage`; past K
+  // load q (0 .. LOADS - 1) of the rows, or of the weight rows, of slice kt into buffer `stage`; past K
   // it is still issued, out of range (only the per-lane offset is checked), and moves nothing
   auto issue_rows = [&](int kt, int stage, int q) {
-    load_to_lds(arsrc, kt < nk ? oa[q] : OUT_OF_RANGE, (unsigned)kt * (BIG_BK * 2), wave_base + stage * BIG_A_BYTES + q * 8192);
+    load_to_lds(arsrc, kt < nk ? oa[q] : OUT_OF_RANGE, (unsigned)kt * (BIG_BK * 2), wave_base + stage * BIG_A_BYTES + q * (WAVES * 1024));
   };
   auto issue_weights = [&](int kt, int stage, int q) {
     load_to_lds(brsrc, kt < nk ? ob[q] : OUT_OF_RANGE, (unsigned)kt * (BIG_BK * 2),
-                wave_base + BIG_A_STAGES * BIG_A_BYTES + stage * BIG_B_BYTES + q * 8192);
+                wave_base + BIG_A_STAGES * BIG_A_BYTES + stage * BIG_B_BYTES + q * (WAVES * 1024));
   };
-  static_assert(BIG_LOADS == 4, "oa and ob hold four loads per wavefront, slice and operand");
 
-  // ---- wavefront tile: rows wm * 128 .. + 128, weight rows brow[0] .. + 32 and brow[1] .. + 32
-  const int wm = wave >> 2, wn = wave & 3;
+  // ---- wavefront tile: the 32-row blocks wm, wm + 2, wm + 4, wm + 6 (so that the two wavefronts
+  // that share weight rows split a short tile's live blocks evenly), weight rows
+  // brow[j] .. + 32 (with SwiGLU the first
+  // half of them gate rows and the second half the up rows of the same columns)
+  const int wm = wave / WN, wn = wave % WN;
   const int l32 = lane & 31;
-  int brow[2];
-  brow[0] = SWIGLU ? wn * 32 : wn * 64;
-  brow[1] = SWIGLU ? COLS + wn * 32 : wn * 64 + 32;
+  int brow[NB];
+#pragma unroll
+  for (int j = 0; j < NB; ++j)
+    brow[j] = SWIGLU ? (j < NB / 2 ? 0 : COLS) + wn * (NB / 2 * 32) + (j % (NB / 2)) * 32 : wn * (NB * 32) + j * 32;
   // byte offset inside a row of K-step s (16 halves = chunks 2s and 2s + 1; the upper 32 lanes
   // take the second); every 32-row block starts at a multiple of 32, so the swizzle depends on
   // the lane alone
@@ -387,45 +392,45 @@ gemm_big_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, co
 #pragma unroll
   for (int s = 0; s < BIG_STEPS; ++s) koff[s] = (((2 * s + (lane >> 5)) ^ ((l32 >> 1) & 7)) * 16);
 
-  float16_t acc[4][2];
+  float16_t acc[4][NB];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < NB; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  const char* as = lds + (wm * 128 + l32) * BIG_ROW_BYTES;
+  const char* as = lds + (wm * 32 + l32) * BIG_ROW_BYTES;
   const char* bs = lds + BIG_A_STAGES * BIG_A_BYTES + l32 * BIG_ROW_BYTES;
 
   // The K loop for LIVE live row blocks (a compile-time count: the loop body is branch-free).
   auto k_loop = [&](auto live_blocks) {
     constexpr int LIVE = decltype(live_blocks)::value;
-    constexpr int READS = LIVE > 0 ? LIVE + 2 : 0, MFMAS = 2 * LIVE;
+    constexpr int READS = LIVE > 0 ? LIVE + NB : 0, MFMAS = NB * LIVE;
     constexpr int PAIRS = READS < MFMAS ? READS : MFMAS;
-    half8_t xf[2][LIVE > 0 ? LIVE : 1], wf[2][2];  // operands of even and odd K-steps
-    // operand r of K-step s of the slice whose rows start at byte sa and weights at sb: the two
+    half8_t xf[2][LIVE > 0 ? LIVE : 1], wf[2][NB];  // operands of even and odd K-steps
+    // operand r of K-step s of the slice whose rows start at byte sa and weights at sb: the
     // weight blocks, then the row blocks
     auto read = [&](int sa, int sb, int s, int r) {
-      if (r < 2) wf[s & 1][r] = *reinterpret_cast<const half8_t*>(bs + sb + brow[r] * BIG_ROW_BYTES + koff[s]);
-      else xf[s & 1][r - 2] = *reinterpret_cast<const half8_t*>(as + sa + (r - 2) * 32 * BIG_ROW_BYTES + koff[s]);
+      if (r < NB) wf[s & 1][r] = *reinterpret_cast<const half8_t*>(bs + sb + brow[r] * BIG_ROW_BYTES + koff[s]);
+      else xf[s & 1][r - NB] = *reinterpret_cast<const half8_t*>(as + sa + (r - NB) * 64 * BIG_ROW_BYTES + koff[s]);
     };
     auto mfma = [&](int s, int m) {
-      const int i = m >> 1, j = m & 1;
+      const int i = m / NB, j = m % NB;
       acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[s & 1][j], xf[s & 1][i], acc[i][j], 0, 0, 0);
     };
     // issue order: rows 0, weights 0 | rows 1, weights 1 | weights 2; from then on rows i + 2
-    // and then weights i + 3, so that "slice i + 1 has landed" is always "all but the last 4"
+    // and then weights i + 3, so that "slice i + 1 has landed" is always "all but the last LOADS"
 #pragma unroll
     for (int p = 0; p < 2; ++p) {
 #pragma unroll
-      for (int q = 0; q < BIG_LOADS; ++q) issue_rows(p, p, q);
+      for (int q = 0; q < LOADS; ++q) issue_rows(p, p, q);
 #pragma unroll
-      for (int q = 0; q < BIG_LOADS; ++q) issue_weights(p, p, q);
+      for (int q = 0; q < LOADS; ++q) issue_weights(p, p, q);
     }
 #pragma unroll
-    for (int q = 0; q < BIG_LOADS; ++q) issue_weights(2, 2, q);
-    asm volatile("s_waitcnt vmcnt(12)" ::: "memory");  // slice 0 has landed
+    for (int q = 0; q < LOADS; ++q) issue_weights(2, 2, q);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * LOADS) : "memory");  // slice 0 has landed
     __syncthreads();
 #pragma unroll
     for (int r = 0; r < READS; ++r) read(0, 0, 0, r);
@@ -454,28 +459,27 @@ gemm_big_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, co
       __builtin_amdgcn_sched_barrier(0);
       // slice kt + 1 has landed (the weights of slice kt + 2 may be out) and this wavefront's
       // reads of slice kt are complete
-      asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
-      static_assert(BIG_LOADS == 4, "the count in the wait above");
+      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(LOADS) : "memory");
       __syncthreads();
-      // the last step in eight parts, each followed by one load: rows kt + 2, then weights kt + 3
+      // the last step in parts, each followed by one load: rows kt + 2, then weights kt + 3
 #pragma unroll
-      for (int part = 0; part < 2 * BIG_LOADS; ++part) {
+      for (int part = 0; part < 2 * LOADS; ++part) {
 #pragma unroll
         for (int r = 0; r < READS; ++r)
-          if (r * 2 * BIG_LOADS / (READS > 0 ? READS : 1) == part) read(a_next * BIG_A_BYTES, b_next * BIG_B_BYTES, 0, r);
+          if (r * 2 * LOADS / (READS > 0 ? READS : 1) == part) read(a_next * BIG_A_BYTES, b_next * BIG_B_BYTES, 0, r);
 #pragma unroll
         for (int m = 0; m < MFMAS; ++m)
-          if (m * 2 * BIG_LOADS / (MFMAS > 0 ? MFMAS : 1) == part) mfma(BIG_STEPS - 1, m);
+          if (m * 2 * LOADS / (MFMAS > 0 ? MFMAS : 1) == part) mfma(BIG_STEPS - 1, m);
         __builtin_amdgcn_sched_barrier(0);
-        if (part < BIG_LOADS) issue_rows(kt + 2, a_stage, part);
-        else issue_weights(kt + 3, b_stage, part - BIG_LOADS);
+        if (part < LOADS) issue_rows(kt + 2, a_stage, part);
+        else issue_weights(kt + 3, b_stage, part - LOADS);
         __builtin_amdgcn_sched_barrier(0);
       }
       a_stage = a_next;
       b_stage = b_next;
     }
   };
-  const int live = max(0, min(4, (nrows - wm * 128 + 31) / 32));
+  const int live = ((nrows + 31) / 32 + 1 - wm) / 2;  // of the tile's live blocks, those this wavefront owns
   switch (live) {
     case 4: k_loop(std::integral_constant<int, 4>{}); break;
     case 3: k_loop(std::integral_constant<int, 3>{}); break;
@@ -489,14 +493,14 @@ gemm_big_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, co
   const int chalf = (lane >> 5) * 4;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int row = row0 + wm * 128 + i * 32 + l32;
+    const int row = row0 + (2 * i + wm) * 32 + l32;
     if (row >= row_end) continue;
     const float sc_row = SCALE ? (float)scale[row] : 1.f;
     half_t* crow = C + (size_t)row * Nout;
-    constexpr int NJ = SWIGLU ? 1 : 2;
+    constexpr int NJ = SWIGLU ? NB / 2 : NB;  // blocks of 32 output columns
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
-      const int cbase = n0 + (SWIGLU ? wn * 32 : wn * 64 + j * 32) + chalf;
+      const int cbase = n0 + wn * (NJ * 32) + j * 32 + chalf;
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int c0 = cbase + 8 * q;
@@ -504,7 +508,7 @@ gemm_big_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, co
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const float v = acc[i][j][4 * q + r];
-          if (SWIGLU) o[r] = swiglu_f16(v, acc[i][1][4 * q + r]);
+          if (SWIGLU) o[r] = swiglu_f16(v, acc[i][SWIGLU ? j + NB / 2 : j][4 * q + r]);
           else if (SCALE) o[r] = (half_t)((float)(half_t)v * sc_row);
           else o[r] = (half_t)v;
         }
@@ -520,6 +524,7 @@ gemm_big_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, co
   }
 }
 
+template <int WN>
 int launch_gemm_big(const half_t* a, const int32_t* a_rows, const half_t* b, const int32_t* offsets, int E, int rows,
                     int Nout, int K, int swiglu, const half_t* s, half_t* c, hipStream_t st) {
   const int cols = swiglu ? BW / 2 : BW;
@@ -527,14 +532,14 @@ int launch_gemm_big(const half_t* a, const int32_t* a_rows, const half_t* b, con
   const long max_row_tiles = rows / BIG_BM + (E < rows ? E : rows);
   const long total = max_row_tiles * ncol_tiles;
   if (total >= (1l << 31) - XCDS) return sy_fail(SY_ERR_ARG, "grouped_gemm: too many tiles");
-  const int per_xcd = (int)((total + XCDS - 1) / XCDS) + 1;  // full and ragged tiles are each rounded up to 8
+  const int per_xcd = (int)((total + XCDS - 1) / XCDS);
   const int grid = per_xcd * XCDS;
   if (swiglu)
-    gemm_big_kernel<true, false><<<grid, BIG_THREADS, 0, st>>>(a, a_rows, b, offsets, E, Nout, K, nullptr, c, ncol_tiles);
+    gemm_big_kernel<WN, true, false><<<grid, 2 * WN * WAVE, 0, st>>>(a, a_rows, b, offsets, E, Nout, K, nullptr, c, ncol_tiles);
   else if (s)
-    gemm_big_kernel<false, true><<<grid, BIG_THREADS, 0, st>>>(a, a_rows, b, offsets, E, Nout, K, s, c, ncol_tiles);
+    gemm_big_kernel<WN, false, true><<<grid, 2 * WN * WAVE, 0, st>>>(a, a_rows, b, offsets, E, Nout, K, s, c, ncol_tiles);
   else
-    gemm_big_kernel<false, false><<<grid, BIG_THREADS, 0, st>>>(a, a_rows, b, offsets, E, Nout, K, nullptr, c, ncol_tiles);
+    gemm_big_kernel<WN, false, false><<<grid, 2 * WN * WAVE, 0, st>>>(a, a_rows, b, offsets, E, Nout, K, nullptr, c, ncol_tiles);
   return sy_check_launch("grouped_gemm");
 }
 
@@ -548,7 +553,7 @@ int launch_gemm(const half_t* a, const int32_t* a_rows, const half_t* b, const i
   const long max_row_tiles = rows / BM + (E < rows ? E : rows);
   const long total = max_row_tiles * ncol_tiles;
   if (total >= (1l << 31) - XCDS) return sy_fail(SY_ERR_ARG, "grouped_gemm: too many tiles");
-  const int per_xcd = (int)((total + XCDS - 1) / XCDS) + 1;  // full and ragged tiles are each rounded up to 8
+  const int per_xcd = (int)((total + XCDS - 1) / XCDS);
   const int grid = per_xcd * XCDS;
   if (swiglu)
     gemm_kernel<MI, true, false><<<grid, GEMM_THREADS, 0, st>>>(a, a_rows, b, offsets, E, Nout, K, nullptr, c, ncol_tiles);
@@ -579,10 +584,9 @@ extern "C" SY_API int sy_grouped_gemm(const void* A, const int32_t* a_rows, cons
   const half_t* b = (const half_t*)B;
   const half_t* s = (const half_t*)scale;
   half_t* c = (half_t*)C;
-  static const int forced = getenv("SY_GEMM_TILE") ? atoi(getenv("SY_GEMM_TILE")) : 0;
-  const int tile = forced ? forced : typical <= 64 ? 64 : typical <= 192 ? 128 : 256;  // 256 needs K % 64 == 0, else 128
-  if (tile == 256 && K % BIG_BK == 0)
-    return launch_gemm_big(a, a_rows, b, offsets, E, rows, Nout, K, swiglu, s, c, (hipStream_t)stream);
+  // measured on 64 experts, 2048 x 1024: the 256-row tile wins from about 128 rows per expert on
+  const int tile = typical <= 64 ? 64 : (typical <= 128 || K % BIG_BK) ? 128 : 256;
+  if (tile == 256) return launch_gemm_big<4>(a, a_rows, b, offsets, E, rows, Nout, K, swiglu, s, c, (hipStream_t)stream);
   if (tile == 64) return launch_gemm<1>(a, a_rows, b, offsets, E, rows, Nout, K, swiglu, s, c, (hipStream_t)stream);
   return launch_gemm<2>(a, a_rows, b, offsets, E, rows, Nout, K, swiglu, s, c, (hipStream_t)stream);
 }

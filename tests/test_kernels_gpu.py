@@ -210,6 +210,41 @@ def test_grouped_kernels_plain_and_ragged_columns(K, fn, swiglu):
     assert (got - want).abs().max().item() < 1e-2
 
 
+@pytest.mark.parametrize("swiglu", [True, False])
+@pytest.mark.parametrize("counts,K_,Nout", [
+    ([40, 0, 64, 1, 33, 90], 64, 72),               # about 38 rows per expert: the 64-row tile
+    ([100, 128, 0, 97, 60, 129], 96, 200),          # about 86: the 128-row tile
+    ([300, 0, 257, 1, 512, 130, 256, 31], 64, 72),  # about 186: the 256-row tile, one K slice
+    ([300, 0, 257, 1, 512, 130, 256, 31], 128, 300),     # two K slices, fewer than the loads in flight
+    ([300, 0, 257, 1, 512, 130, 256, 31], 448, 256),     # seven slices
+    ([300, 0, 257, 1, 512, 130, 256, 31], 96, 128),      # K % 64 != 0: falls back to the 128-row tile
+    ([1500, 2, 700], 192, 136),                     # many row tiles per expert, ragged columns
+])
+def test_grouped_gemm_every_tile_kind(K, counts, K_, Nout, swiglu):
+    """Gathered rows, per-row scale (plain projection) or SwiGLU, experts with 0, 1 and many rows:
+    grouped_gemm picks its tile from the mean rows per expert, so the shapes walk through all
+    three tile kinds and the short-K corners of the one that keeps several slices in flight."""
+    E, rows = len(counts), sum(counts)
+    g = torch.Generator().manual_seed(rows + K_)
+    src = torch.randn(rows // 2 + 3, K_, generator=g).half()
+    a_rows = torch.randint(0, src.shape[0], (rows,), generator=g).int()
+    B = (torch.randn(E, Nout * (2 if swiglu else 1), K_, generator=g) * K_ ** -0.5).half()
+    scale = None if swiglu else torch.rand(rows, generator=g).half()
+    offsets = torch.zeros(E + 1, dtype=torch.int32)
+    offsets[1:] = torch.cumsum(torch.tensor(counts), 0)
+    got = K.ext().grouped_gemm(src.to(DEV), a_rows.to(DEV), B.to(DEV), offsets.to(DEV), None, 0, rows, swiglu,
+                               None if scale is None else scale.to(DEV)).float().cpu()
+    A = src[a_rows.long()]
+    want = torch.empty(rows, Nout)
+    for e in range(E):
+        s, t = int(offsets[e]), int(offsets[e + 1])
+        r = F.linear(A[s:t].float(), B[e].float())
+        want[s:t] = F.silu(r[:, :Nout].half().float()).half().float() * r[:, Nout:].half().float() if swiglu \
+            else r.half().float() * scale[s:t, None].float()
+    assert got.shape == (rows, Nout)
+    assert (got - want).abs().max().item() < 1e-2
+
+
 # ------------------------------------------------------------------ the layer, the reference's test
 @pytest.mark.parametrize("N", [1, 7, 64, 333, 2048])
 @pytest.mark.parametrize("skew", [0.0, 2.0])
