@@ -1,10 +1,10 @@
 // combine: each token's k expert outputs summed in fp32, in ascending expert id, rounded to
 // f16 once.
 //
-// One workgroup per token. The first k threads rank the token's choices by (expert id, slot)
-// and leave the k source rows in LDS in that order; then every thread owns 16-byte columns
-// of the output and adds the k rows in order, so the result does not depend on the launch
-// shape.
+// One workgroup per token. The first wavefront loads the token's k ids and rows together, ranks
+// the choices by (expert id, slot) with lane reads and leaves the k source rows in LDS in that
+// order; then every thread owns 16-byte columns of the output and adds the k rows in order, so
+// the result does not depend on the launch shape.
 //
 // Replaces combine_kernel / combine of the reference (switchyard/csrc/moe_kernels.cu:417-444).
 #include "common.h"
@@ -17,16 +17,17 @@ constexpr int MAX_K = 64;
 __global__ void __launch_bounds__(COMBINE_THREADS)
 combine_kernel(const half_t* __restrict__ y, const int* __restrict__ pos_of, const int* __restrict__ idx, int k, int H,
                half_t* __restrict__ out) {
-  __shared__ int ids[MAX_K];
   __shared__ int rows[MAX_K];
   const int t = blockIdx.x, tid = threadIdx.x;
-  if (tid < k) ids[tid] = idx[(size_t)t * k + tid];
-  __syncthreads();
-  if (tid < k) {
-    const int mine = ids[tid];
+  if (tid < WAVE) {
+    const int mine = tid < k ? idx[(size_t)t * k + tid] : 0x7fffffff;
+    const int row = tid < k ? pos_of[(size_t)t * k + tid] : 0;
     int rank = 0;
-    for (int j = 0; j < k; ++j) rank += (ids[j] < mine) || (ids[j] == mine && j < tid);
-    rows[rank] = pos_of[(size_t)t * k + tid];
+    for (int j = 0; j < k; ++j) {
+      const int other = read_lane(mine, j);
+      rank += (other < mine) || (other == mine && j < tid);
+    }
+    if (tid < k) rows[rank] = row;
   }
   __syncthreads();
   for (int c = tid * 8; c < H; c += COMBINE_THREADS * 8) {

@@ -16,7 +16,6 @@ namespace {
 using namespace sort_core;
 
 constexpr int FRONT_THREADS = SORT_THREADS;  // 1024: the sort wants 16 wavefronts
-constexpr int FRONT_WAVES = FRONT_THREADS / WAVE;
 constexpr int FRONT_MAX_TOKENS = 256;
 constexpr int FRONT_MAX_K = 8;
 
@@ -32,7 +31,7 @@ front_kernel(const half_t* __restrict__ logits, int N, int E, int k, int norm, i
   const int M = N * k;
   int* sidx = lds + small_sort_lds_ints(E);
   half_t* sw = reinterpret_cast<half_t*>(sidx + M);
-  for (int t = wave; t < N; t += FRONT_WAVES) {
+  for (int t = wave; t < N; t += (int)(blockDim.x >> 6)) {
     int my_e;
     float my_w;
     route_core::route_token<half_t, PER_LANE>(logits + (size_t)t * E, E, k, norm, my_e, my_w);
@@ -46,7 +45,13 @@ front_kernel(const half_t* __restrict__ logits, int N, int E, int k, int norm, i
   }
   __syncthreads();
 
-  // ---- sort
+  // ---- sort: at most one choice per lane of one wavefront, or the workgroup's counting sort
+  if (M <= WAVE) {
+    if (wave == 0)
+      sort_one_wave<uint16_t>(sidx, reinterpret_cast<const uint16_t*>(sw), M, k, E, nbits, counts, offsets, token,
+                              reinterpret_cast<uint16_t*>(wsorted), pos_of, lds);
+    return;
+  }
   sort_small_block<uint16_t>(sidx, reinterpret_cast<const uint16_t*>(sw), M, k, E, nbits, counts, offsets, token,
                              reinterpret_cast<uint16_t*>(wsorted), pos_of, lds);
 }
@@ -65,11 +70,13 @@ extern "C" SY_API int sy_route_sort(const void* logits, int N, int E, int k, int
   const int M = N * k;
   const size_t lds = sizeof(int) * (small_sort_lds_ints(E) + M) + sizeof(half_t) * M;
   hipStream_t st = (hipStream_t)stream;
+  // one wavefront per token is all that the route needs when one wavefront sorts
+  const int threads = M <= WAVE ? N * WAVE : FRONT_THREADS;
   if (E <= 64)
-    front_kernel<1><<<1, FRONT_THREADS, lds, st>>>((const half_t*)logits, N, E, k, norm, nbits, idx, (half_t*)w, counts,
+    front_kernel<1><<<1, threads, lds, st>>>((const half_t*)logits, N, E, k, norm, nbits, idx, (half_t*)w, counts,
                                                   offsets, token, (half_t*)wsorted, pos_of);
   else
-    front_kernel<2><<<1, FRONT_THREADS, lds, st>>>((const half_t*)logits, N, E, k, norm, nbits, idx, (half_t*)w, counts,
+    front_kernel<2><<<1, threads, lds, st>>>((const half_t*)logits, N, E, k, norm, nbits, idx, (half_t*)w, counts,
                                                   offsets, token, (half_t*)wsorted, pos_of);
   return sy_check_launch("route_sort");
 }

@@ -123,5 +123,49 @@ __device__ __forceinline__ void sort_small_block(const int* idx, const W* w, int
   assign_piece(idx, w, lo, hi, k, E, nbits, hist + wv * E, token, wsorted, pos_of);
 }
 
+// The whole sort by one wavefront when there are at most 64 choices (a decode step of 8 tokens):
+// one choice per lane, no workgroup barrier. `lds` holds 2 * E + 1 ints; E <= 128.
+template <typename W>
+__device__ __forceinline__ void sort_one_wave(const int* idx, const W* w, int M, int k, int E, int nbits,
+                                              int* __restrict__ counts, int* __restrict__ offsets,
+                                              int* __restrict__ token, W* __restrict__ wsorted,
+                                              int* __restrict__ pos_of, int* lds) {
+  int* total = lds;      // [E]
+  int* offs = lds + E;   // [E + 1]
+  const int lane = threadIdx.x & 63;
+  for (int x = lane; x < E; x += WAVE) total[x] = 0;
+  int key = lane < M ? idx[lane] : -1;
+  const bool valid = (unsigned)key < (unsigned)E;
+  key = valid ? key : 0;
+  const uint64_t m = match_lanes(key, valid, nbits);
+  const int rank = __popcll(m & lanemask_lt()), cnt = __popcll(m);
+  __builtin_amdgcn_wave_barrier();
+  if (valid && rank == cnt - 1) total[key] = cnt;  // one lane per expert
+  __builtin_amdgcn_wave_barrier();
+  int run = 0;
+  for (int x0 = 0; x0 < E; x0 += WAVE) {
+    const int x = x0 + lane;
+    const int c = x < E ? total[x] : 0;
+    int inc = c;
+    for (int o = 1; o < WAVE; o <<= 1) {
+      const int up = __shfl_up(inc, o, WAVE);
+      if (lane >= o) inc += up;
+    }
+    if (x < E) {
+      counts[x] = c;
+      offsets[x] = run + inc - c;
+      offs[x] = run + inc - c;
+    }
+    run += __shfl(inc, WAVE - 1, WAVE);
+  }
+  if (lane == 0) offsets[E] = run;
+  __builtin_amdgcn_wave_barrier();
+  if (valid) {
+    const int row = offs[key] + rank;
+    token[row] = lane / k;
+    wsorted[row] = w[lane];
+    pos_of[lane] = row;
+  }
+}
 
 }  // namespace sort_core
