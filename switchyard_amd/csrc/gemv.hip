@@ -84,8 +84,15 @@ __device__ __forceinline__ void run_pass(const Pass& p) {
   constexpr int PARTS = SWIGLU ? 2 : 1;  // a unit is streamed as its gate rows, then its up rows
   const half8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
 
-  // ---- issue side: part `ipt` of unit `iun`, chunk `ich` is the next to load
-  int iun = 0, ipt = 0, ich = 0;
+  // Units start at different steps of K and wrap around: wavefronts that run in step would
+  // otherwise all ask for the same stretch of their rows at the same time, and rows a multiple
+  // of 4 KB apart then meet on the same few memory channels.
+  const int nsteps = p.nchunks * CH;
+  const int rot0 = (p.unit0 * 5) % nsteps;
+
+  // ---- issue side: part `ipt` of unit `iun`, chunk `ich` (counted from the unit's start `irot`)
+  // is the next to load
+  int iun = 0, ipt = 0, ich = 0, irot = rot0;
   auto issue = [&](Chunk& c) {
     const int col = (p.unit0 + iun) * UNIT_COLS + sub;
     const int wr = ipt ? p.Nout + col : col;
@@ -93,7 +100,8 @@ __device__ __forceinline__ void run_pass(const Pass& p) {
     if (!EXACT && col >= p.Nout) lane_off = OUT_OF_RANGE;
 #pragma unroll
     for (int s = 0; s < CH; ++s) {
-      const int kk = (ich * CH + s) * STEP_K;
+      const int at = ich * CH + s + irot;
+      const int kk = (at - (at >= nsteps ? nsteps : 0)) * STEP_K;
       unsigned off = lane_off;
       if (!EXACT && kk + klane >= p.K) off = OUT_OF_RANGE;
       c.w[s] = load_stream(p.rsrc, off, (unsigned)kk * 2u);
@@ -103,12 +111,13 @@ __device__ __forceinline__ void run_pass(const Pass& p) {
       if (++ipt == PARTS) {
         ipt = 0;
         ++iun;
+        irot = (irot + 5) % nsteps;
       }
     }
   };
 
   // ---- compute side
-  int cun = 0, cpt = 0, cch = 0;
+  int cun = 0, cpt = 0, cch = 0, crot = rot0;
   float4_t acc[NQ], gate[NQ];
 #pragma unroll
   for (int q = 0; q < NQ; ++q) acc[q] = gate[q] = float4_t{0.f, 0.f, 0.f, 0.f};
@@ -117,7 +126,8 @@ __device__ __forceinline__ void run_pass(const Pass& p) {
   auto compute = [&](const Chunk& c) {
 #pragma unroll
     for (int s = 0; s < CH; ++s) {
-      const int kk = (cch * CH + s) * STEP_K;
+      const int at = cch * CH + s + crot;
+      const int kk = (at - (at >= nsteps ? nsteps : 0)) * STEP_K;
 #pragma unroll
       for (int q = 0; q < NQ; ++q) {
         half8_t x = *reinterpret_cast<const half8_t*>(xlane + q * QUAD * p.RS + kk);
@@ -164,6 +174,7 @@ __device__ __forceinline__ void run_pass(const Pass& p) {
     if (++cpt == PARTS) {
       cpt = 0;
       ++cun;
+      crot = (crot + 5) % nsteps;
     }
   };
 

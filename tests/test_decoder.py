@@ -117,18 +117,35 @@ def test_random_weights_have_the_loader_layout():
 @pytest.mark.parametrize("batch", [2, 8])
 def test_kernel_hook_decodes_the_same_tokens_as_the_loop_hook(batch):
     """fp16 on the GPU: hook = HIP kernels against hook = per-expert loop (oracle) on the same
-    weights. Identical greedy tokens, identical top-1 of the first logits, close logits."""
+    weights. The first logits agree to 2e-2 with the same top-1; every token the kernels'
+    greedy decode picks is the loop model's top-1 for the same prefix, up to ties inside the
+    logits tolerance (a random-init model has near-equal logits, and the two hooks round their
+    fp16 sums in different orders); where the loop model's margin is clear the pick is the same."""
     s = D.Shape(vocab=1000, hidden=512, intermediate=256, layers=4, heads=8, kv_heads=8, head_dim=64, experts=64, top_k=8)
     w = D.random_weights(s, device="cuda", seed=1, std=0.05)
     ps = [torch.randint(3, s.vocab, (24 + 3 * b,), generator=torch.Generator().manual_seed(b)).tolist()
           for b in range(batch)]
     fast = D.Decoder(s, w, max_positions=128)
     slow = D.Decoder(s, w, moe=loop_hook(s, w), max_positions=128)
-    a, la = fast.generate(ps, 16, return_first_logits=True)
-    b, lb = slow.generate(ps, 16, return_first_logits=True)
-    assert torch.equal(la.argmax(-1), lb.argmax(-1))
-    assert (la.float() - lb.float()).abs().max().item() < 2e-2
-    assert a == b
+    new = 16
+    a, la = fast.generate(ps, new, return_first_logits=True)
+    _, lb = slow.generate(ps, new, return_first_logits=True)
+    tol = 2e-2
+    assert (la.float() - lb.float()).abs().max().item() < tol
+    clear = lb.float().topk(2, -1).values
+    clear = (clear[:, 0] - clear[:, 1]) > 2 * tol
+    assert torch.equal(la.argmax(-1)[clear], lb.argmax(-1)[clear])
+    checked = 0  # positions with a clear margin (informational: a random-init model has few)
+    for prompt, picked in zip(ps, a):
+        seq = torch.tensor([prompt + picked], device="cuda")
+        logits = slow.forward(seq)[0, len(prompt) - 1:len(prompt) - 1 + len(picked)].float()
+        best = logits.max(-1).values
+        chosen = logits.gather(1, torch.tensor(picked, device="cuda")[:, None])[:, 0]
+        assert (best - chosen).max().item() <= 2 * tol, "a picked token is not the loop model's top-1 within tolerance"
+        top2 = logits.topk(2, -1).values
+        sure = (top2[:, 0] - top2[:, 1]) > 2 * tol
+        assert torch.equal(logits.argmax(-1)[sure].cpu(), torch.tensor(picked)[sure.cpu()])
+        checked += int(sure.sum())
 
 
 @pytest.mark.gpu
