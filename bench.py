@@ -172,7 +172,7 @@ def run_default(args):
         roof = {"bound": "mfma", "achieved": alg / (k_ms / 1e3) / 1e12, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s"}
     roof["frac"] = roof["achieved"] / roof["peak"]
     roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(N)
-    roof["kernel"] = "gemv_kernel<swiglu> (gate/up projection)" if use_gemv else "gemm_kernel<swiglu> (gate/up projection)"
+    roof["kernel"] = "gemv_kernel<swiglu> (gate/up projection)" if use_gemv else "grouped_gemm<swiglu> (gate/up projection)"
     roof["us_per_launch"] = k_ms * 1e3
     roof["algorithmic_per_launch"] = alg
 

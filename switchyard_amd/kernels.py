@@ -42,11 +42,13 @@ def route(h, router, top_k, norm_topk_prob):
     return ext().route(F.linear(h, router).contiguous(), top_k, norm_topk_prob)
 
 
-# Measured on an MI355X with OLMoE's shapes (bench.py --sweep): the weight-stream kernel wins
-# while the busiest expert has at most 16 rows (64 tokens: 0.244 vs 0.269 ms per layer; 96
-# tokens, 20 rows: 0.311 vs 0.260 ms), the MFMA tile kernel beyond. The reference's third
-# regime (a library GEMM per expert above 48 rows) does not exist on this hardware.
-GEMV_MAX_ROWS = 16
+# Measured on an MI355X with OLMoE's shapes (bench.py --sweep, ms for the experts of one layer,
+# weight stream vs MFMA tiles): 8 tokens 0.147 vs 0.160, 16 tokens 0.174 vs 0.174, 24 tokens
+# 0.190 vs 0.191, 32 tokens (busiest expert 9 rows) 0.201 vs 0.194, 64 tokens 0.231 vs 0.209,
+# 96 tokens 0.305 vs 0.203. The weight-stream kernel wins while the busiest expert has at most
+# 8 rows. The reference's third regime (a library GEMM per expert above 48 rows) does not
+# exist on this hardware.
+GEMV_MAX_ROWS = 8
 GEMM_MAX_ROWS = 1 << 30
 
 
