@@ -22,6 +22,19 @@ int sy_check_launch(const char* what) {
   return sy_fail(SY_ERR_LAUNCH, "%s: launch failed: %s", what, hipGetErrorString(err));
 }
 
+// Compute units of the current device (cached per device id; read-only after the first call).
+int sy_compute_units() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
 extern "C" SY_API int sy_version(void) { return 100; }
 
 extern "C" SY_API const char* sy_last_error(void) { return g_error; }

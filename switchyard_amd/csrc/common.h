@@ -21,6 +21,9 @@ int sy_fail(int code, const char* fmt, ...);
 // Returns SY_OK, or records the pending HIP launch error and returns SY_ERR_LAUNCH.
 int sy_check_launch(const char* what);
 
+// Compute units of the current device (cached per device).
+int sy_compute_units();
+
 #define SY_REQUIRE(cond, ...) \
   do {                        \
     if (!(cond)) return sy_fail(SY_ERR_ARG, __VA_ARGS__); \

@@ -312,6 +312,11 @@ __device__ __forceinline__ int4_t buffer_descriptor(const void* base, unsigned b
 // 16 bytes per lane from buffer offset voffset + soffset to LDS address lds_addr + 16 * lane.
 // Only voffset is checked against the size of the buffer.
 __device__ __forceinline__ void load_to_lds(int4_t rsrc, unsigned voffset, unsigned soffset, unsigned lds_addr) {
+  // the descriptor, the slice offset and the LDS address are the same in every lane; say so
+#pragma unroll
+  for (int c = 0; c < 4; ++c) rsrc[c] = __builtin_amdgcn_readfirstlane(rsrc[c]);
+  soffset = __builtin_amdgcn_readfirstlane(soffset);
+  lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
   asm volatile(
       "s_mov_b32 m0, %0\n\t"
       "s_nop 0\n\t"
@@ -588,6 +593,7 @@ extern "C" SY_API int sy_grouped_gemm(const void* A, const int32_t* a_rows, cons
   SY_REQUIRE(K >= 32 && K % 32 == 0, "grouped_gemm: K must be a multiple of 32 (got %d)", K);
   SY_REQUIRE(!(swiglu && scale), "grouped_gemm: swiglu and scale are not combined");
   SY_REQUIRE((long)Nout * K * (swiglu ? 4 : 2) < (1l << 31), "grouped_gemm: an expert's matrix must stay under 2 GiB");
+  SY_REQUIRE(a_rows || (long)rows * K * 2 < (1l << 31), "grouped_gemm: A must stay under 2 GiB (%d rows of %d)", rows, K);
   if (rows == 0) return SY_OK;
   SY_REQUIRE(A && B && offsets && C, "grouped_gemm: null pointer");
   // rows per tile: 64 while the typical expert fits in one such tile (the launch is then a

@@ -278,19 +278,6 @@ gemv_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const 
   }
 }
 
-// Compute units of the current device (cached per device id; read-only after the first call).
-int compute_units() {
-  static int cached[64] = {0};
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  if (cached[dev] == 0) {
-    int n = 0;
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    cached[dev] = n;
-  }
-  return cached[dev];
-}
-
 int launch_gemv(const void* A, const int32_t* a_rows, const void* B, const int32_t* offsets, int E, int rows,
                 int max_rows_hint, int Nout, int K, int swiglu, const void* scale, void* C, hipStream_t stream) {
   // rows staged per pass: no expert has more rows than there are rows in all; a caller that
@@ -301,7 +288,7 @@ int launch_gemv(const void* A, const int32_t* a_rows, const void* B, const int32
   const size_t lds = (size_t)row_cap * (K + ROW_PAD) * sizeof(half_t) + (size_t)(E + 1) * sizeof(int);
   // persistent: a fixed number of workgroups per CU, but no more than there are units
   const long max_units = (long)(E < rows ? E : rows) * ((Nout + UNIT_COLS - 1) / UNIT_COLS);
-  long grid = (long)compute_units() * BLOCKS_PER_CU;
+  long grid = (long)sy_compute_units() * BLOCKS_PER_CU;
   grid = grid > max_units ? max_units : grid;
   const half_t* a = (const half_t*)A;
   const half_t* b = (const half_t*)B;
