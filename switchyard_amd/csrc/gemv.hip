@@ -42,7 +42,6 @@ constexpr int STEP_K = 128;     // K covered by one load instruction (16 blocks 
 constexpr int CH = 4;           // load steps per chunk
 constexpr int ROW_PAD = 32;     // halves of padding per staged row (64 bytes)
 constexpr int MAX_E = 1024;     // experts whose ids fit the LDS list
-constexpr int BLOCKS_PER_CU = 2;
 
 // 128-bit streaming load through a buffer descriptor: lane offset in bytes (out of range
 // reads return 0), wave-uniform offset in an SGPR.
@@ -286,15 +285,23 @@ int launch_gemv(const void* A, const int32_t* a_rows, const void* B, const int32
   int row_cap = (bound + QUAD - 1) / QUAD * QUAD;
   row_cap = row_cap > MAX_QUADS * QUAD ? MAX_QUADS * QUAD : row_cap;
   const size_t lds = (size_t)row_cap * (K + ROW_PAD) * sizeof(half_t) + (size_t)(E + 1) * sizeof(int);
-  // persistent: a fixed number of workgroups per CU, but no more than there are units
+  const bool exact = K % (CH * STEP_K) == 0 && Nout % UNIT_COLS == 0;
+  // persistent: a fixed number of workgroups per CU, but no more than there are units. Two per
+  // CU stream best when a unit is 32 KB of weights (gate and up rows of 2048: 57.8 us against
+  // 59.0 and 63.4 with three and four), four when it is 8 KB (rows of 1024: 31.8 us against
+  // 32.2 and 33.4 with three and two); all of them must be resident at once.
+  const long unit_bytes = (long)UNIT_COLS * K * 2 * (swiglu ? 2 : 1);
+  long per_cu = unit_bytes >= 32768 ? 2 : unit_bytes >= 16384 ? 3 : 4;
+  if (!exact && per_cu > 3) per_cu = 3;                       // the masked variants need more registers
+  const long fit = (160 * 1024) / (long)(lds ? lds : 1);      // by LDS
+  per_cu = per_cu > fit ? (fit > 0 ? fit : 1) : per_cu;
   const long max_units = (long)(E < rows ? E : rows) * ((Nout + UNIT_COLS - 1) / UNIT_COLS);
-  long grid = (long)sy_compute_units() * BLOCKS_PER_CU;
+  long grid = (long)sy_compute_units() * per_cu;
   grid = grid > max_units ? max_units : grid;
   const half_t* a = (const half_t*)A;
   const half_t* b = (const half_t*)B;
   const half_t* s = (const half_t*)scale;
   half_t* c = (half_t*)C;
-  const bool exact = K % (CH * STEP_K) == 0 && Nout % UNIT_COLS == 0;
   void (*kern)(const half_t*, const int*, const half_t*, const int*, int, int, int, const half_t*, half_t*, int);
   if (swiglu) kern = exact ? gemv_kernel<true, false, true> : gemv_kernel<true, false, false>;
   else if (s) kern = exact ? gemv_kernel<false, true, true> : gemv_kernel<false, true, false>;
