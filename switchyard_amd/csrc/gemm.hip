@@ -1,7 +1,10 @@
 // grouped_gemm: the prefill path. Every expert's slice of the sorted rows goes through that
-// expert's weights on fp16 MFMA tiles, all experts in one launch.
+// expert's weights on fp16 MFMA tiles, all experts in one launch. Three tiles, chosen by the
+// host from the mean rows per expert: 64 or 128 rows (gemm_kernel, below) while the launch is
+// mostly a stream over the weights, 256 rows (gemm_big_kernel, further down) once it is bound
+// by the MFMAs.
 //
-// Tile: 64*MI rows x 256 weight rows (MI = 1 or 2), K in slices of 64, 4 wavefronts, each computing
+// gemm_kernel. Tile: 64*MI rows x 256 weight rows (MI = 1 or 2), K in slices of 64, 4 wavefronts, each computing
 // all of the tile's rows x 64 weight rows as (2*MI) x 2 v_mfma_f32_32x32x16_f16 blocks with fp32
 // accumulators. With SwiGLU the 256 weight rows are 128 gate rows and the 128 up rows of the
 // same output columns, and a wavefront holds gate and up of the same 32 columns, so the
