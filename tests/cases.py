@@ -55,3 +55,12 @@ def weight_bytes(used, H=2048, I=1024):
 
 def layer_flops(M, H=2048, I=1024):
     return M * 6 * H * I
+
+
+def golden_sort_vector():
+    """The reference's own known-answer vector for sort_by_expert (tests/golden/README.md)."""
+    import json
+    import os
+
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "sort_by_expert_reference_vector.json")) as f:
+        return json.load(f)

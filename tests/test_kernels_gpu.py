@@ -125,12 +125,13 @@ def test_sort_is_bit_exact_stable_and_deterministic(K, N, E, k):
 
 
 def test_sort_known_answer_from_the_reference_tests(K):
-    idx = torch.tensor([[2, 0], [0, 1], [2, 1]], dtype=torch.int32, device=DEV)
-    w = torch.tensor([[.6, .4], [.7, .3], [.5, .5]], dtype=torch.float16, device=DEV)
-    counts, offsets, token, wsorted, pos_of = K.ext().sort_by_expert(idx, w, 4)
-    assert counts.tolist() == [2, 2, 2, 0] and offsets.tolist() == [0, 2, 4, 6, 6]
-    assert token.tolist() == [0, 1, 1, 2, 0, 2] and pos_of.tolist() == [4, 0, 1, 2, 5, 3]
-    assert torch.allclose(wsorted.float().cpu(), torch.tensor([.4, .7, .3, .5, .6, .5]), atol=1e-3)
+    g = cases.golden_sort_vector()
+    idx = torch.tensor(g["idx"], dtype=torch.int32, device=DEV)
+    w = torch.tensor(g["w"], dtype=torch.float16, device=DEV)
+    counts, offsets, token, wsorted, pos_of = K.ext().sort_by_expert(idx, w, g["n_experts"])
+    assert counts.tolist() == g["counts"] and offsets.tolist() == g["offsets"]
+    assert token.tolist() == g["token"] and pos_of.tolist() == g["pos_of"]
+    assert torch.allclose(wsorted.float().cpu(), torch.tensor(g["weight"]), atol=1e-3)
 
 
 def test_sort_with_repeats_skew_and_fp32_weights(K):

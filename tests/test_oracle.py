@@ -6,6 +6,7 @@ import pytest
 import torch
 import torch.nn.functional as F
 
+import cases
 from oracle import c_oracle
 from oracle import moe_oracle as O
 
@@ -13,26 +14,25 @@ from oracle import moe_oracle as O
 # ------------------------------------------------------------------ sort / plan
 def test_plan_known_answer_from_the_reference_tests():
     # The literal vector of the reference's tests/test_model.py:49-57; pos_of by ep.py:40-41.
-    idx = torch.tensor([[2, 0], [0, 1], [2, 1]])
-    w = torch.tensor([[.6, .4], [.7, .3], [.5, .5]])
-    p = O.plan(idx, w, 4)
-    assert p.counts.tolist() == [2, 2, 2, 0]
-    assert p.offsets.tolist() == [0, 2, 4, 6, 6]
-    assert p.token.tolist() == [0, 1, 1, 2, 0, 2]
-    assert p.slot.tolist() == [1, 0, 1, 1, 0, 0]
-    assert torch.allclose(p.weight, torch.tensor([.4, .7, .3, .5, .6, .5]))
-    assert p.pos_of.tolist() == [4, 0, 1, 2, 5, 3]
+    g = cases.golden_sort_vector()
+    p = O.plan(torch.tensor(g["idx"]), torch.tensor(g["w"]), g["n_experts"])
+    assert p.counts.tolist() == g["counts"]
+    assert p.offsets.tolist() == g["offsets"]
+    assert p.token.tolist() == g["token"]
+    assert p.slot.tolist() == g["slot"]
+    assert torch.allclose(p.weight, torch.tensor(g["weight"]))
+    assert p.pos_of.tolist() == g["pos_of"]
 
 
 def test_c_sort_known_answer_from_the_reference_tests():
-    idx = np.array([[2, 0], [0, 1], [2, 1]], dtype=np.int32)
-    w = np.array([[.6, .4], [.7, .3], [.5, .5]], dtype=np.float32)
-    counts, offsets, token, wsorted, pos_of = c_oracle.sort_by_expert(idx, w, 4)
-    assert counts.tolist() == [2, 2, 2, 0]
-    assert offsets.tolist() == [0, 2, 4, 6, 6]
-    assert token.tolist() == [0, 1, 1, 2, 0, 2]
-    assert np.allclose(wsorted, [.4, .7, .3, .5, .6, .5])
-    assert pos_of.tolist() == [4, 0, 1, 2, 5, 3]
+    g = cases.golden_sort_vector()
+    counts, offsets, token, wsorted, pos_of = c_oracle.sort_by_expert(
+        np.array(g["idx"], dtype=np.int32), np.array(g["w"], dtype=np.float32), g["n_experts"])
+    assert counts.tolist() == g["counts"]
+    assert offsets.tolist() == g["offsets"]
+    assert token.tolist() == g["token"]
+    assert np.allclose(wsorted, g["weight"])
+    assert pos_of.tolist() == g["pos_of"]
 
 
 @pytest.mark.parametrize("N,k,E", [(1, 8, 64), (37, 8, 64), (300, 4, 60), (64, 2, 8), (500, 8, 128), (5, 3, 200)])
