@@ -212,6 +212,31 @@ def test_grouped_kernels_plain_and_ragged_columns(K, fn, swiglu):
 
 
 @pytest.mark.parametrize("swiglu", [True, False])
+def test_grouped_gemv_with_many_experts(K, swiglu):
+    """150 experts with 0 to 5 rows each: the list of used experts spans several 64-lane scans."""
+    E, K_, Nout = 150, 256, 24
+    counts = torch.tensor([(3 * i) % 6 for i in range(E)])
+    rows = int(counts.sum())
+    g = torch.Generator().manual_seed(3)
+    src = torch.randn(40, K_, generator=g).half()
+    a_rows = torch.randint(0, 40, (rows,), generator=g).int()
+    B = (torch.randn(E, Nout * (2 if swiglu else 1), K_, generator=g) * K_ ** -0.5).half()
+    scale = None if swiglu else torch.rand(rows, generator=g).half()
+    offsets = torch.zeros(E + 1, dtype=torch.int32)
+    offsets[1:] = torch.cumsum(counts, 0)
+    got = K.ext().grouped_gemv(src.to(DEV), a_rows.to(DEV), B.to(DEV), offsets.to(DEV), rows, swiglu,
+                               None if scale is None else scale.to(DEV)).float().cpu()
+    A = src[a_rows.long()]
+    want = torch.empty(rows, Nout)
+    for e in range(E):
+        s, t = int(offsets[e]), int(offsets[e + 1])
+        r = F.linear(A[s:t].float(), B[e].float())
+        want[s:t] = F.silu(r[:, :Nout].half().float()).half().float() * r[:, Nout:].half().float() if swiglu \
+            else r.half().float() * scale[s:t, None].float()
+    assert (got - want).abs().max().item() < 1e-2
+
+
+@pytest.mark.parametrize("swiglu", [True, False])
 @pytest.mark.parametrize("counts,K_,Nout", [
     ([40, 0, 64, 1, 33, 90], 64, 72),               # about 38 rows per expert: the 64-row tile
     ([100, 128, 0, 97, 60, 129], 96, 200),          # about 86: the 128-row tile
@@ -220,6 +245,8 @@ def test_grouped_kernels_plain_and_ragged_columns(K, fn, swiglu):
     ([300, 0, 257, 1, 512, 130, 256, 31], 448, 256),     # seven slices
     ([300, 0, 257, 1, 512, 130, 256, 31], 96, 128),      # K % 64 != 0: falls back to the 128-row tile
     ([1500, 2, 700], 192, 136),                     # many row tiles per expert, ragged columns
+    ([(7 * i) % 23 for i in range(150)], 64, 40),         # 150 experts (several 64-lane scans), about 11 rows each
+    ([((11 * i) % 7) * 90 for i in range(130)], 128, 264),   # 130 experts, 0 to 540 rows: the 256-row tile
 ])
 def test_grouped_gemm_every_tile_kind(K, counts, K_, Nout, swiglu):
     """Gathered rows, per-row scale (plain projection) or SwiGLU, experts with 0, 1 and many rows:
@@ -243,7 +270,8 @@ def test_grouped_gemm_every_tile_kind(K, counts, K_, Nout, swiglu):
         want[s:t] = F.silu(r[:, :Nout].half().float()).half().float() * r[:, Nout:].half().float() if swiglu \
             else r.half().float() * scale[s:t, None].float()
     assert got.shape == (rows, Nout)
-    assert (got - want).abs().max().item() < 1e-2
+    # one rounding to f16 of differently ordered fp32 sums: an absolute floor plus half-precision ulps
+    assert torch.allclose(got, want, rtol=2.0 ** -9, atol=1e-2)
 
 
 # ------------------------------------------------------------------ the layer, the reference's test
