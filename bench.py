@@ -269,8 +269,15 @@ def run_decode(args):
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    s = D.OLMOE_1B_7B
-    w = D.random_weights(s, device=dev, seed=0)
+    if args.checkpoint:
+        from switchyard_amd import checkpoint as C
+        s, _ = C.shape_from_config(args.checkpoint)
+        w = C.load(args.checkpoint, s, dtype=torch.float16, device=dev)
+        name = f"checkpoint {args.checkpoint}, {s.layers} layers, fp16"
+    else:
+        s = D.OLMOE_1B_7B
+        w = D.random_weights(s, device=dev, seed=0)
+        name = "OLMoE-1B-7B shape, 16 layers, random-init fp16"
     model = D.Decoder(s, w, max_positions=args.prompt_len + args.new_tokens + 8)
 
     def loop_moe(i, h):
@@ -310,7 +317,7 @@ def run_decode(args):
                "top1_rows_identical_to_loop_hook": int(agree.sum()), "rows": B,
                "largest_loop_hook_margin_where_top1_differs": float(margin[~agree].max()) if (~agree).any() else 0.0,
                "first_logits_max_abs_diff": (first.float() - ref_first.float()).abs().max().item(),
-               "model": "OLMoE-1B-7B shape, 16 layers, random-init fp16", "gpu": torch.cuda.get_device_name(0)}
+               "model": name, "gpu": torch.cuda.get_device_name(0)}
         if args.decode_loop_steps:
             cache = D.KVCache(s, B, args.prompt_len + args.decode_loop_steps, torch.float16, dev)
             logits = loop_model.forward(tokens, cache)[:, -1]
@@ -338,6 +345,8 @@ def main():
                          "rocprofv3's FETCH_SIZE / WRITE_SIZE readings)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg (profiling runs)")
     ap.add_argument("--decode", default=None, help='full-model greedy decode at these batch sizes, e.g. "8,64"')
+    ap.add_argument("--checkpoint", default=None,
+                    help="decode: an OLMoE checkpoint directory (config.json + safetensors) instead of random weights")
     ap.add_argument("--prompt-len", type=int, default=512)
     ap.add_argument("--new-tokens", type=int, default=128)
     ap.add_argument("--decode-loop-steps", type=int, default=8,
