@@ -1,0 +1,61 @@
+/* switchyard_decode.h: C ABI of the decode-step kernels in libswitchyard_moe.so that sit around
+ * the MoE layer: the attention side of one step of the decoder that calls the MoE hook, when
+ * every sequence of the batch advances by one token. They replace the PyTorch operator
+ * sequences of the reference's switchyard/model.py named at each entry point; the projections
+ * between them (wq/wk/wv stacked, wo, lm_head) go through sy_grouped_gemv / sy_grouped_gemm of
+ * switchyard_moe.h with one "expert". Conventions as in switchyard_moe.h: device pointers
+ * borrowed for the call, caller-allocated outputs, `stream` a hipStream_t, f16 row-major
+ * tensors, 0 or an SY_ERR_* code returned, no state kept, nothing allocated.
+ * The cache slot and the rotary positions are read from device memory, so a captured HIP
+ * graph of these launches can be replayed for every step.
+ */
+#ifndef SWITCHYARD_DECODE_H
+#define SWITCHYARD_DECODE_H
+
+#include "switchyard_moe.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Residual add and RMS norm in one pass; replaces `x = x + delta` followed by rmsnorm()
+ * (switchyard/model.py:14-17 as used at :119-121,142 and :130).
+ * x, delta f16 [N,H] (delta may be NULL: no add); weight f16 [H] ->
+ * x_out f16 [N,H] = f16(x + delta) (may be x itself, or NULL to skip the store),
+ * h_out f16 [N,H] = weight * f16(x_out * rsqrt(mean(x_out^2) + eps)), the mean in fp32.
+ * Limits: H % 8 == 0, H <= 8192. N == 0 is a no-op. */
+SY_API int sy_add_rmsnorm(const void* x, const void* delta, const void* weight, float eps, int N, int H, void* x_out,
+                          void* h_out, void* stream);
+
+/* What follows the q/k/v projections of one new token per sequence; replaces the rmsnorm of q
+ * and k, the clamp, the rotary embedding and the cache write of _attention()
+ * (switchyard/model.py:64-77) with T = 1.
+ * qkv f16 [B, (heads + 2*kv_heads)*D]: a row holds q, then k, then v; q_norm f16 [heads*D],
+ * k_norm f16 [kv_heads*D] (the norm runs over the whole projection, not per head);
+ * clip > 0 clamps q, k and v to [-clip, clip]; cos_table, sin_table f16 [max_positions, D]
+ * (both halves of a row equal, as cat([freqs, freqs])); positions int64 [B] rotary position of
+ * each sequence's new token; slot int64 [1] cache position to write (the same for every
+ * sequence of a left-padded batch) ->
+ * q_out f16 [B, heads*D]; kcache, vcache f16 [B, kv_heads, capacity, D] get the new key and
+ * value at [:, :, slot, :]. A slot outside [0, capacity) writes nothing.
+ * Limits: D % 16 == 0, heads*D <= 8192, heads % kv_heads == 0. B == 0 is a no-op. */
+SY_API int sy_qk_norm_rope_cache(const void* qkv, const void* q_norm, const void* k_norm, float eps, float clip,
+                                 const void* cos_table, const void* sin_table, int max_positions,
+                                 const int64_t* positions, const int64_t* slot, int B, int heads, int kv_heads, int D,
+                                 int capacity, void* q_out, void* kcache, void* vcache, void* stream);
+
+/* One query per (sequence, head) against the KV cache; replaces the scores / mask / softmax /
+ * value product of _attention() (switchyard/model.py:78-84) with T = 1.
+ * q f16 [B, heads*D]; kcache, vcache f16 [B, kv_heads, capacity, D]; real uint8 [B, capacity]
+ * (0 where the cache position holds left padding); slot int64 [1]: keys 0..slot are visible ->
+ * out f16 [B, heads*D] = softmax(q.k / sqrt(D)) v over the visible real keys (fp32 inside);
+ * zeros if a sequence has none. Query head h reads kv head h / (heads / kv_heads).
+ * Limits: D is 64 or 128. B == 0 is a no-op. */
+SY_API int sy_decode_attention(const void* q, const void* kcache, const void* vcache, const uint8_t* real,
+                               const int64_t* slot, int B, int heads, int kv_heads, int D, int capacity, void* out,
+                               void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SWITCHYARD_DECODE_H */

@@ -1,4 +1,5 @@
-"""ctypes binding of libswitchyard_moe.so (C ABI in include/switchyard_moe.h).
+"""ctypes binding of libswitchyard_moe.so (C ABI in include/switchyard_moe.h and, for the
+decode-step kernels around the MoE layer, include/switchyard_decode.h).
 
 `Ext` offers the functions of the reference's pybind module `switchyard_moe`
 (switchyard/csrc/moe_kernels.cu:491-500) with the same names, argument order and results,
@@ -16,9 +17,9 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libswitchyard_moe.so")
 
-_c_int, _c_void_p, _c_size_t = ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t
+_c_int, _c_void_p, _c_size_t, _c_float = ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_float
 
-# name -> (restype, argtypes); mirrors include/switchyard_moe.h
+# name -> (restype, argtypes); mirrors include/switchyard_moe.h and include/switchyard_decode.h
 SIGNATURES = {
     "sy_version": (_c_int, []),
     "sy_last_error": (ctypes.c_char_p, []),
@@ -33,6 +34,13 @@ SIGNATURES = {
     "sy_grouped_gemm": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int,
                                  _c_void_p, _c_void_p, _c_void_p]),
     "sy_combine": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p]),
+    "sy_add_rmsnorm": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_int, _c_int, _c_void_p, _c_void_p,
+                                _c_void_p]),
+    "sy_qk_norm_rope_cache": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_float, _c_void_p, _c_void_p, _c_int,
+                                       _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p,
+                                       _c_void_p, _c_void_p, _c_void_p]),
+    "sy_decode_attention": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
+                                     _c_int, _c_int, _c_void_p, _c_void_p]),
 }
 
 
@@ -171,4 +179,71 @@ class Ext:
         out = torch.empty((n_tokens, H), dtype=y.dtype, device=y.device)
         self._call(self.lib.sy_combine, y.data_ptr(), pos_of.data_ptr(), idx.data_ptr(), int(n_tokens), k, H,
                    out.data_ptr(), _stream())
+        return out
+
+    # ---- the decode-step kernels around the MoE layer (include/switchyard_decode.h)
+    def add_rmsnorm(self, x, delta, weight, eps, x_out=None):
+        """x [N, H] (+ delta [N, H] or None) -> (x + delta, weight * rmsnorm(x + delta)).
+        With delta None the first result is x itself; x_out may be x for an update in place."""
+        _check(x, "x", torch.float16)
+        _check(weight, "weight", torch.float16)
+        N, H = x.shape
+        if weight.numel() != H:
+            raise RuntimeError("add_rmsnorm: weight must have H entries")
+        if delta is not None:
+            _check(delta, "delta", torch.float16)
+            if delta.shape != x.shape:
+                raise RuntimeError("add_rmsnorm: delta must have x's shape")
+            if x_out is None:
+                x_out = torch.empty_like(x)
+            _check(x_out, "x_out", torch.float16)
+            if x_out.shape != x.shape:
+                raise RuntimeError("add_rmsnorm: x_out must have x's shape")
+        h = torch.empty_like(x)
+        self._call(self.lib.sy_add_rmsnorm, x.data_ptr(), delta.data_ptr() if delta is not None else None,
+                   weight.data_ptr(), float(eps), N, H, x_out.data_ptr() if delta is not None else None, h.data_ptr(),
+                   _stream())
+        return (x_out if delta is not None else x), h
+
+    def qk_norm_rope_cache(self, qkv, q_norm, k_norm, eps, clip, cos, sin, positions, slot, heads, kv_heads, head_dim,
+                           kcache, vcache):
+        """qkv [B, (heads + 2 kv_heads) D] -> q [B, heads D] normed and rotated; the new key and
+        value go into kcache / vcache [B, kv_heads, capacity, D] at the device-held `slot`."""
+        for t, name in ((qkv, "qkv"), (q_norm, "q_norm"), (k_norm, "k_norm"), (cos, "cos"), (sin, "sin"),
+                        (kcache, "kcache"), (vcache, "vcache")):
+            _check(t, name, torch.float16)
+        _check(positions, "positions", torch.int64)
+        _check(slot, "slot", torch.int64)
+        B, D = qkv.shape[0], int(head_dim)
+        if qkv.shape[1] != (heads + 2 * kv_heads) * D or q_norm.numel() != heads * D or k_norm.numel() != kv_heads * D:
+            raise RuntimeError("qk_norm_rope_cache: qkv / q_norm / k_norm do not match heads, kv_heads and head_dim")
+        if cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] != D:
+            raise RuntimeError("qk_norm_rope_cache: cos and sin must be [max_positions, head_dim]")
+        if kcache.shape != vcache.shape or kcache.dim() != 4 or tuple(kcache.shape[:2]) != (B, kv_heads) or \
+                kcache.shape[3] != D:
+            raise RuntimeError("qk_norm_rope_cache: caches must be [B, kv_heads, capacity, head_dim]")
+        if positions.numel() != B or slot.numel() != 1:
+            raise RuntimeError("qk_norm_rope_cache: positions [B] and slot [1]")
+        q = torch.empty((B, heads * D), dtype=torch.float16, device=qkv.device)
+        self._call(self.lib.sy_qk_norm_rope_cache, qkv.data_ptr(), q_norm.data_ptr(), k_norm.data_ptr(), float(eps),
+                   float(clip or 0.0), cos.data_ptr(), sin.data_ptr(), cos.shape[0], positions.data_ptr(),
+                   slot.data_ptr(), B, int(heads), int(kv_heads), D, kcache.shape[2], q.data_ptr(), kcache.data_ptr(),
+                   vcache.data_ptr(), _stream())
+        return q
+
+    def decode_attention(self, q, kcache, vcache, real, slot, heads):
+        """q [B, heads D] against kcache / vcache [B, kv_heads, capacity, D], keys 0..slot that
+        `real` [B, capacity] (bool) marks -> [B, heads D]."""
+        _check(q, "q", torch.float16)
+        _check(kcache, "kcache", torch.float16)
+        _check(vcache, "vcache", torch.float16)
+        _check(real, "real", torch.bool)
+        _check(slot, "slot", torch.int64)
+        B, kv_heads, capacity, D = kcache.shape
+        if vcache.shape != kcache.shape or tuple(q.shape) != (B, heads * D) or tuple(real.shape) != (B, capacity) or \
+                slot.numel() != 1:
+            raise RuntimeError("decode_attention: shapes of q / caches / real / slot do not match")
+        out = torch.empty_like(q)
+        self._call(self.lib.sy_decode_attention, q.data_ptr(), kcache.data_ptr(), vcache.data_ptr(), real.data_ptr(),
+                   slot.data_ptr(), B, int(heads), kv_heads, D, capacity, out.data_ptr(), _stream())
         return out

@@ -12,7 +12,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libswitchyard_moe.so")
-SOURCES = ["abi.hip", "route.hip", "sort.hip", "front.hip", "combine.hip", "gemv.hip", "gemm.hip"]
+SOURCES = ["abi.hip", "route.hip", "sort.hip", "front.hip", "combine.hip", "gemv.hip", "gemm.hip", "decode.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
     # hipcc -O3 must not form packed fp32 instructions from scalar float code

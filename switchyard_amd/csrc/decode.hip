@@ -1,0 +1,366 @@
+// The attention side of one decode step, for the caller of the MoE hook: what sits between two
+// MoE layers when every sequence of the batch advances by one token. In the reference this is
+// a few dozen PyTorch launches per layer (switchyard/model.py:14-17 rmsnorm, :61-84
+// _attention, :117-121 attention_block); at decode each of them is a launch that moves a few
+// kilobytes, so the step is bound by launches, not by the 34 MB of attention weights and the
+// KV cache it has to read. Three kernels replace them (the projections themselves go through
+// the weight-stream kernel with a single "expert"):
+//
+//   add_rmsnorm           x += delta; h = w * f16(x * rsqrt(mean(x^2) + eps))       (one row per workgroup)
+//   qk_norm_rope_cache    q/k RMS norm over the whole projection, clamp, rotary embedding, and
+//                         the new key and value written into the cache at `slot`
+//   decode_attention      one query per (sequence, head) against the cache: a single pass over
+//                         the keys and values with a running softmax, HBM-bound
+//
+// Everything a replayed HIP graph must not bake in (the cache slot, the rotary positions) is
+// read from device memory, so the same launches serve every step.
+//
+// Rounding follows the PyTorch graph on fp16 tensors where it is cheap to do so: the norm is
+// taken in fp32, rounded to fp16 and then scaled in fp16; rotary products and their sum are
+// each rounded to fp16. Attention scores and the softmax stay in fp32 (the reference rounds
+// the scores to fp16 first), which is the more exact of the two.
+#include "common.h"
+#include "../../include/switchyard_decode.h"
+
+namespace {
+
+constexpr int ROW_THREADS = 256;
+constexpr int MAX_CHUNKS = 4;  // 8-half chunks per thread: rows of up to 8192 halves
+
+__device__ __forceinline__ float block_sum(float v, float* lds, int slot_base) {
+  // sum over the 4 wavefronts of a 256-thread workgroup; every thread gets the total
+  v = wave_sum(v);
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) lds[slot_base + wave] = v;
+  __syncthreads();
+  return lds[slot_base] + lds[slot_base + 1] + lds[slot_base + 2] + lds[slot_base + 3];
+}
+
+__global__ void __launch_bounds__(ROW_THREADS)
+add_rmsnorm_kernel(const half_t* x, const half_t* __restrict__ delta, const half_t* __restrict__ weight, float eps,
+                   int H, half_t* x_out, half_t* __restrict__ h_out) {  // x_out may be x
+  __shared__ float part[4];
+  const size_t row = (size_t)blockIdx.x * H;
+  const int chunks = H >> 3;
+  half8_t v[MAX_CHUNKS];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < MAX_CHUNKS; ++i) {
+    const int c = threadIdx.x + i * ROW_THREADS;
+    if (c < chunks) {
+      v[i] = *reinterpret_cast<const half8_t*>(x + row + c * 8);
+      if (delta) {
+        const half8_t d = *reinterpret_cast<const half8_t*>(delta + row + c * 8);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[i][j] = (half_t)((float)v[i][j] + (float)d[j]);
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ss += (float)v[i][j] * (float)v[i][j];
+    }
+  }
+  const float rs = rsqrtf(block_sum(ss, part, 0) / (float)H + eps);
+#pragma unroll
+  for (int i = 0; i < MAX_CHUNKS; ++i) {
+    const int c = threadIdx.x + i * ROW_THREADS;
+    if (c < chunks) {
+      const half8_t w = *reinterpret_cast<const half8_t*>(weight + c * 8);
+      half8_t h;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) h[j] = (half_t)((float)w[j] * (float)(half_t)((float)v[i][j] * rs));
+      if (x_out) *reinterpret_cast<half8_t*>(x_out + row + c * 8) = v[i];
+      *reinterpret_cast<half8_t*>(h_out + row + c * 8) = h;
+    }
+  }
+}
+
+__device__ __forceinline__ half_t clamp_f16(half_t v, float clip) {
+  if (clip > 0.f) {
+    const float f = (float)v;
+    return (half_t)(f < -clip ? -clip : f > clip ? clip : f);
+  }
+  return v;
+}
+
+// out = f16(f16(y * cos) + f16(rot * sin)): three roundings, as three PyTorch operators on
+// fp16 tensors make them. Contraction is switched off here, or the compiler narrows the
+// arithmetic to fp16 and fuses product and sum into one fma with a single rounding.
+__device__ __forceinline__ half_t rotary_f16(half_t y, half_t rot, half_t cos_v, half_t sin_v) {
+#pragma clang fp contract(off)
+  const half_t t1 = (half_t)((float)y * (float)cos_v);
+  const half_t t2 = (half_t)((float)rot * (float)sin_v);
+  return (half_t)((float)t1 + (float)t2);
+}
+
+// One workgroup per sequence. qkv row = [q (heads*D) | k (kv_heads*D) | v (kv_heads*D)].
+__global__ void __launch_bounds__(ROW_THREADS)
+qk_norm_rope_cache_kernel(const half_t* __restrict__ qkv, const half_t* __restrict__ q_norm,
+                          const half_t* __restrict__ k_norm, float eps, float clip, const half_t* __restrict__ cos_t,
+                          const half_t* __restrict__ sin_t, int max_positions, const int64_t* __restrict__ positions,
+                          const int64_t* __restrict__ slot_ptr, int heads, int kv_heads, int D, int capacity,
+                          half_t* __restrict__ q_out, half_t* __restrict__ kcache, half_t* __restrict__ vcache) {
+  extern __shared__ __attribute__((aligned(16))) half_t normed[];  // [qd + kvd] after norm and clamp
+  __shared__ float part[8];
+  const int b = blockIdx.x;
+  const int qd = heads * D, kvd = kv_heads * D;
+  const half_t* row = qkv + (size_t)b * (qd + 2 * kvd);
+  const int qchunks = qd >> 3, kchunks = kvd >> 3;
+  const long slot = (long)*slot_ptr;
+  long pos = (long)positions[b];
+  pos = pos < 0 ? 0 : pos >= max_positions ? max_positions - 1 : pos;
+  const bool slot_ok = slot >= 0 && slot < capacity;
+
+  half8_t q[MAX_CHUNKS], k[MAX_CHUNKS];
+  float sq = 0.f, sk = 0.f;
+#pragma unroll
+  for (int i = 0; i < MAX_CHUNKS; ++i) {
+    const int c = threadIdx.x + i * ROW_THREADS;
+    if (c < qchunks) {
+      q[i] = *reinterpret_cast<const half8_t*>(row + c * 8);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) sq += (float)q[i][j] * (float)q[i][j];
+    }
+    if (c < kchunks) {
+      k[i] = *reinterpret_cast<const half8_t*>(row + qd + c * 8);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) sk += (float)k[i][j] * (float)k[i][j];
+    }
+  }
+  const float rq = rsqrtf(block_sum(sq, part, 0) / (float)qd + eps);
+  const float rk = rsqrtf(block_sum(sk, part, 4) / (float)kvd + eps);
+#pragma unroll
+  for (int i = 0; i < MAX_CHUNKS; ++i) {
+    const int c = threadIdx.x + i * ROW_THREADS;
+    if (c < qchunks) {
+      const half8_t w = *reinterpret_cast<const half8_t*>(q_norm + c * 8);
+      half8_t o;
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        o[j] = clamp_f16((half_t)((float)w[j] * (float)(half_t)((float)q[i][j] * rq)), clip);
+      *reinterpret_cast<half8_t*>(normed + c * 8) = o;
+    }
+    if (c < kchunks) {
+      const half8_t w = *reinterpret_cast<const half8_t*>(k_norm + c * 8);
+      half8_t o;
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        o[j] = clamp_f16((half_t)((float)w[j] * (float)(half_t)((float)k[i][j] * rk)), clip);
+      *reinterpret_cast<half8_t*>(normed + qd + c * 8) = o;
+    }
+  }
+  __syncthreads();
+
+  // rotary embedding: out[d] = f16(y[d] * cos[d]) + f16(rot[d] * sin[d]), rot = [-y[D/2:], y[:D/2]]
+  const int half_d = D >> 1;
+  const half_t* cs = cos_t + (size_t)pos * D;
+  const half_t* sn = sin_t + (size_t)pos * D;
+  const int all = qchunks + kchunks;
+  for (int c = threadIdx.x; c < all; c += ROW_THREADS) {
+    const int d0 = (c * 8) % D;  // qd is a multiple of D, so this also holds in the k part
+    const half8_t y = *reinterpret_cast<const half8_t*>(normed + c * 8);
+    const bool low = d0 < half_d;
+    const half8_t other = *reinterpret_cast<const half8_t*>(normed + c * 8 + (low ? half_d : -half_d));
+    const half8_t cc = *reinterpret_cast<const half8_t*>(cs + d0);
+    const half8_t ssn = *reinterpret_cast<const half8_t*>(sn + d0);
+    half8_t o;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      o[j] = rotary_f16(y[j], low ? -other[j] : other[j], cc[j], ssn[j]);
+    }
+    if (c < qchunks) {
+      *reinterpret_cast<half8_t*>(q_out + (size_t)b * qd + c * 8) = o;
+    } else if (slot_ok) {
+      const int e = (c - qchunks) * 8, h = e / D;
+      *reinterpret_cast<half8_t*>(kcache + (((size_t)b * kv_heads + h) * capacity + slot) * D + (e - h * D)) = o;
+    }
+  }
+  if (slot_ok) {
+    for (int c = threadIdx.x; c < kchunks; c += ROW_THREADS) {
+      half8_t v = *reinterpret_cast<const half8_t*>(row + qd + kvd + c * 8);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = clamp_f16(v[j], clip);
+      const int e = c * 8, h = e / D;
+      *reinterpret_cast<half8_t*>(vcache + (((size_t)b * kv_heads + h) * capacity + slot) * D + (e - h * D)) = v;
+    }
+  }
+}
+
+// Sum over the LPK lanes that share a key (LPK = 16: one DPP row; 8: half a row).
+template <int LPK>
+__device__ __forceinline__ float key_sum(float v) {
+  if (LPK == 16) return row_allreduce(v, [](float a, float b) { return a + b; });
+  v += __shfl_xor(v, 4, WAVE);
+  v += __shfl_xor(v, 2, WAVE);
+  v += __shfl_xor(v, 1, WAVE);
+  return v;
+}
+
+constexpr int ATT_UNROLL = 4;        // key groups in flight per wavefront
+constexpr float MASKED = -1.0e30f;   // running maximum before any key was seen
+
+// One workgroup per (sequence, query head), NW wavefronts. A load instruction covers KPL =
+// 64 / LPK consecutive keys (LPK = D / 8 lanes per key, 16 bytes per lane: whole 256-byte rows
+// for D = 128), so the cache is read as long contiguous runs. Each group of LPK lanes keeps its
+// own running softmax (maximum, sum, 8 output dimensions per lane) over the keys it meets, so
+// the key loop has no cross-lane traffic except the score's sum; the KPL x NW partial results
+// are merged once at the end.
+template <int LPK>
+__global__ void decode_attention_kernel(const half_t* __restrict__ q, const half_t* __restrict__ kcache,
+                                        const half_t* __restrict__ vcache, const uint8_t* __restrict__ real,
+                                        const int64_t* __restrict__ slot_ptr, int heads, int kv_heads, int capacity,
+                                        float scale_log2e, half_t* __restrict__ out) {
+  constexpr int D = LPK * 8, KPL = WAVE / LPK;
+  extern __shared__ float merge[];  // [NW][D + 2]: accumulators, maximum, sum
+  const int NW = blockDim.x >> 6;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int sub = lane / LPK, c = lane % LPK;
+  const int b = blockIdx.x / heads, qh = blockIdx.x % heads;
+  const int kvh = qh / (heads / kv_heads);
+  long n = (long)*slot_ptr + 1;
+  n = n < 0 ? 0 : n > capacity ? capacity : n;
+
+  const half8_t qv = *reinterpret_cast<const half8_t*>(q + ((size_t)b * heads + qh) * D + c * 8);
+  float qf[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) qf[j] = (float)qv[j] * scale_log2e;
+  const size_t base = ((size_t)b * kv_heads + kvh) * (size_t)capacity * D + c * 8;
+  const uint8_t* rl = real + (size_t)b * capacity;
+
+  float m = MASKED, l = 0.f, acc[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+  const half8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  const int groups = ((int)n + KPL - 1) / KPL;
+  for (int g0 = wave; g0 < groups; g0 += NW * ATT_UNROLL) {
+    half8_t kk[ATT_UNROLL], vv[ATT_UNROLL];
+    bool ok[ATT_UNROLL];
+#pragma unroll
+    for (int u = 0; u < ATT_UNROLL; ++u) {
+      const int key = (g0 + u * NW) * KPL + sub;
+      ok[u] = key < n;
+      kk[u] = zero8;
+      vv[u] = zero8;
+      if (ok[u]) {
+        kk[u] = *reinterpret_cast<const half8_t*>(kcache + base + (size_t)key * D);
+        vv[u] = *reinterpret_cast<const half8_t*>(vcache + base + (size_t)key * D);
+        ok[u] = rl[key] != 0;
+      }
+    }
+    float s[ATT_UNROLL], mx = m;
+#pragma unroll
+    for (int u = 0; u < ATT_UNROLL; ++u) {
+      float d = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) d += qf[j] * (float)kk[u][j];
+      s[u] = key_sum<LPK>(d);
+      if (ok[u]) mx = fmaxf(mx, s[u]);
+    }
+    const float alpha = __builtin_amdgcn_exp2f(m - mx);
+    m = mx;
+    l *= alpha;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] *= alpha;
+#pragma unroll
+    for (int u = 0; u < ATT_UNROLL; ++u) {
+      const float p = ok[u] ? __builtin_amdgcn_exp2f(s[u] - mx) : 0.f;
+      l += p;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[j] += p * (float)vv[u][j];
+    }
+  }
+
+  // ---- merge the KPL key groups of the wavefront (lanes with equal c)
+  float mw = m;
+#pragma unroll
+  for (int off = LPK; off < WAVE; off <<= 1) mw = fmaxf(mw, __shfl_xor(mw, off, WAVE));
+  const float a = __builtin_amdgcn_exp2f(m - mw);
+  l *= a;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) acc[j] *= a;
+#pragma unroll
+  for (int off = LPK; off < WAVE; off <<= 1) {
+    l += __shfl_xor(l, off, WAVE);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] += __shfl_xor(acc[j], off, WAVE);
+  }
+  float* mine = merge + wave * (D + 2);
+  if (sub == 0) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) mine[c * 8 + j] = acc[j];
+    if (c == 0) {
+      mine[D] = mw;
+      mine[D + 1] = l;
+    }
+  }
+  __syncthreads();
+  // ---- merge the wavefronts: thread d < D finishes output dimension d
+  if (threadIdx.x < D) {
+    float M = MASKED;
+    for (int w = 0; w < NW; ++w) M = fmaxf(M, merge[w * (D + 2) + D]);
+    float num = 0.f, den = 0.f;
+    for (int w = 0; w < NW; ++w) {
+      const float f = __builtin_amdgcn_exp2f(merge[w * (D + 2) + D] - M);
+      num += f * merge[w * (D + 2) + threadIdx.x];
+      den += f * merge[w * (D + 2) + D + 1];
+    }
+    out[((size_t)b * heads + qh) * D + threadIdx.x] = (half_t)(den > 0.f ? num / den : 0.f);
+  }
+}
+
+}  // namespace
+
+extern "C" SY_API int sy_add_rmsnorm(const void* x, const void* delta, const void* weight, float eps, int N, int H,
+                                     void* x_out, void* h_out, void* stream) {
+  SY_REQUIRE(N >= 0 && H >= 8 && H % 8 == 0 && H <= 8 * ROW_THREADS * MAX_CHUNKS,
+             "add_rmsnorm: N = %d, H = %d (a multiple of 8 up to %d)", N, H, 8 * ROW_THREADS * MAX_CHUNKS);
+  if (N == 0) return SY_OK;
+  SY_REQUIRE(x && weight && h_out, "add_rmsnorm: null pointer");
+  add_rmsnorm_kernel<<<N, ROW_THREADS, 0, (hipStream_t)stream>>>((const half_t*)x, (const half_t*)delta,
+                                                                 (const half_t*)weight, eps, H, (half_t*)x_out,
+                                                                 (half_t*)h_out);
+  return sy_check_launch("add_rmsnorm");
+}
+
+extern "C" SY_API int sy_qk_norm_rope_cache(const void* qkv, const void* q_norm, const void* k_norm, float eps, float clip,
+                                            const void* cos_table, const void* sin_table, int max_positions,
+                                            const int64_t* positions, const int64_t* slot, int B, int heads,
+                                            int kv_heads, int D, int capacity, void* q_out, void* kcache, void* vcache,
+                                            void* stream) {
+  SY_REQUIRE(B >= 0 && heads >= 1 && kv_heads >= 1 && heads % kv_heads == 0,
+             "qk_norm_rope_cache: B = %d, heads = %d, kv_heads = %d", B, heads, kv_heads);
+  SY_REQUIRE(D >= 16 && D % 16 == 0 && (long)heads * D <= 8 * ROW_THREADS * MAX_CHUNKS,
+             "qk_norm_rope_cache: head_dim = %d must be a multiple of 16 and heads * head_dim at most %d", D,
+             8 * ROW_THREADS * MAX_CHUNKS);
+  SY_REQUIRE(capacity >= 1 && max_positions >= 1, "qk_norm_rope_cache: capacity = %d, max_positions = %d", capacity,
+             max_positions);
+  if (B == 0) return SY_OK;
+  SY_REQUIRE(qkv && q_norm && k_norm && cos_table && sin_table && positions && slot && q_out && kcache && vcache,
+             "qk_norm_rope_cache: null pointer");
+  const size_t lds = (size_t)(heads + kv_heads) * D * sizeof(half_t);
+  qk_norm_rope_cache_kernel<<<B, ROW_THREADS, lds, (hipStream_t)stream>>>(
+      (const half_t*)qkv, (const half_t*)q_norm, (const half_t*)k_norm, eps, clip, (const half_t*)cos_table,
+      (const half_t*)sin_table, max_positions, positions, slot, heads, kv_heads, D, capacity, (half_t*)q_out,
+      (half_t*)kcache, (half_t*)vcache);
+  return sy_check_launch("qk_norm_rope_cache");
+}
+
+extern "C" SY_API int sy_decode_attention(const void* q, const void* kcache, const void* vcache, const uint8_t* real,
+                                          const int64_t* slot, int B, int heads, int kv_heads, int D, int capacity,
+                                          void* out, void* stream) {
+  SY_REQUIRE(B >= 0 && heads >= 1 && kv_heads >= 1 && heads % kv_heads == 0,
+             "decode_attention: B = %d, heads = %d, kv_heads = %d", B, heads, kv_heads);
+  SY_REQUIRE(D == 64 || D == 128, "decode_attention: head_dim must be 64 or 128 (got %d)", D);
+  SY_REQUIRE(capacity >= 1, "decode_attention: capacity = %d", capacity);
+  if (B == 0) return SY_OK;
+  SY_REQUIRE(q && kcache && vcache && real && slot && out, "decode_attention: null pointer");
+  // few (sequence, head) pairs: 16 wavefronts each, so that the cache is still read by many
+  const long pairs = (long)B * heads;
+  const int waves = pairs >= 2l * sy_compute_units() ? 4 : 16;
+  const size_t lds = (size_t)waves * (D + 2) * sizeof(float);
+  const float scale_log2e = 1.4426950408889634f / sqrtf((float)D);
+  auto kern = D == 128 ? decode_attention_kernel<16> : decode_attention_kernel<8>;
+  kern<<<(unsigned)pairs, waves * WAVE, lds, (hipStream_t)stream>>>((const half_t*)q, (const half_t*)kcache,
+                                                                   (const half_t*)vcache, real, slot, heads, kv_heads,
+                                                                   capacity, scale_log2e, (half_t*)out);
+  return sy_check_launch("decode_attention");
+}

@@ -6,9 +6,11 @@ mixture-of-experts layer goes through `moe(layer_index, h[B*T, H]) -> [B*T, H]`,
 default is `kernels.moe_layer` on the layer's router / gate_up / down tensors.
 
 Built for decode on one GPU: the KV cache is allocated once for the whole generation, rotary
-tables are precomputed, attention is one fused scaled-dot-product call, and the greedy loop
-keeps its tokens on the device, so a decode step is a queue of launches with no host read
-unless the caller asks for early stopping at `eos`.
+tables are precomputed, and the greedy loop keeps its tokens on the device, so a decode step
+is a queue of launches with no host read unless the caller asks for early stopping at `eos`.
+On a GPU in fp16 the attention side of a decode step runs on the library's decode kernels
+(`step_fused`: about ten launches per layer with the MoE layer's five, every projection a
+weight stream); prefill, fp32 and the CPU use the PyTorch operators (`forward`, `step_static`).
 """
 
 from dataclasses import dataclass
@@ -125,10 +127,18 @@ class KVCache:
 
 
 class Decoder:
-    def __init__(self, shape, weights, moe=None, max_positions=4096):
+    def __init__(self, shape, weights, moe=None, max_positions=4096, attention="auto"):
+        """attention: "kernels" (the decode kernels for one-token steps), "torch", or "auto":
+        kernels where they apply (GPU, fp16, head_dim 64 or 128)."""
         self.s, self.w = shape, weights
         self.moe = moe or self.kernel_moe
         dev = weights["embed"].device
+        can = (dev.type == "cuda" and weights["embed"].dtype == torch.float16 and shape.head_dim in (64, 128)
+               and shape.hidden % 8 == 0 and shape.hidden <= 8192 and shape.heads * shape.head_dim <= 8192)
+        if attention == "kernels" and not can:
+            raise ValueError("the decode kernels need a GPU, fp16 weights and head_dim 64 or 128")
+        self.fused = can if attention == "auto" else attention == "kernels"
+        self._wqkv = None
         inv = 1.0 / (shape.rope_theta ** (torch.arange(0, shape.head_dim, 2, device=dev).float() / shape.head_dim))
         ang = torch.outer(torch.arange(max_positions, device=dev).float(), inv)
         table = torch.cat([ang, ang], dim=-1)
@@ -235,6 +245,49 @@ class Decoder:
         slot += 1
         return F.linear(_rms(x, W["final_norm"], s.rms_eps), W["lm_head"])[:, -1]
 
+    def _stacked_qkv(self):
+        """wq, wk, wv of every layer stacked as one [q | k | v] projection, so that the three are
+        one weight stream; the dictionary's own entries become views of the stack."""
+        if self._wqkv is None:
+            self._wqkv = []
+            for L in self.w["layers"]:
+                stack = torch.cat([L["wq"], L["wk"], L["wv"]]).contiguous()
+                qd, kvd = L["wq"].shape[0], L["wk"].shape[0]
+                L["wq"], L["wk"], L["wv"] = stack[:qd], stack[qd:qd + kvd], stack[qd + kvd:]
+                self._wqkv.append(stack)
+        return self._wqkv
+
+    @torch.no_grad()
+    def step_fused(self, tok, cache, slot, keys=None):
+        """The same step as `step_static` on the decode kernels: residual add + RMS norm, the
+        stacked q/k/v projection, norm + rotary + cache write, attention over the cache, the
+        output projection, and the MoE hook; every projection streams its weights once."""
+        from . import kernels
+
+        s, W, E = self.s, self.w, kernels.ext()
+        wqkv = self._stacked_qkv()
+        positions = cache.next_position
+        cache.real.index_fill_(1, slot, True)
+        x = F.embedding(tok[:, 0], W["embed"])
+        delta = None
+        for i in range(s.layers):
+            L = W["layers"][i]
+            x, xn = E.add_rmsnorm(x, delta, L["attn_norm"], s.rms_eps, x_out=x)
+            q = E.qk_norm_rope_cache(kernels.dense(xn, wqkv[i]), L["q_norm"], L["k_norm"], s.rms_eps, s.clip_qkv,
+                                     self.cos, self.sin, positions, slot, s.heads, s.kv_heads, s.head_dim,
+                                     cache.k[i], cache.v[i])
+            a = E.decode_attention(q, cache.k[i], cache.v[i], cache.real, slot, s.heads)
+            x, h = E.add_rmsnorm(x, kernels.dense(a, L["wo"]), L["mlp_norm"], s.rms_eps, x_out=x)
+            delta = self.moe(i, h)
+        x, xn = E.add_rmsnorm(x, delta, W["final_norm"], s.rms_eps, x_out=x)
+        cache.next_position += 1
+        slot += 1
+        return kernels.dense(xn, W["lm_head"])
+
+    def step(self, tok, cache, slot, keys):
+        """One decode step for every sequence: tok [B, 1] -> logits [B, vocab]; advances the cache."""
+        return self.step_fused(tok, cache, slot) if self.fused else self.step_static(tok, cache, slot, keys)
+
     @torch.no_grad()
     def generate_graph(self, prompts, max_new_tokens, return_first_logits=False, timings=None):
         """Greedy decoding with the decode step captured once in a HIP graph and replayed per
@@ -268,7 +321,7 @@ class Decoder:
             keys = torch.arange(cache.capacity, device=dev)
 
             def one_token():
-                logits = self.step_static(tok, cache, slot, keys)
+                logits = self.step(tok, cache, slot, keys)
                 tok.copy_(logits.argmax(-1)[:, None])
                 out.index_copy_(1, col, tok)
                 col.add_(1)
@@ -318,6 +371,7 @@ class Decoder:
         out = torch.empty(B, max_new_tokens, dtype=torch.long, device=dev)
         steps = 0
         alive = torch.ones(B, dtype=torch.bool, device=dev)
+        slot = torch.tensor([cache.filled], dtype=torch.long, device=dev) if self.fused else None
         for step in range(max_new_tokens):
             nxt = logits.argmax(-1)
             out[:, step] = nxt
@@ -327,7 +381,11 @@ class Decoder:
                 if not bool(alive.any()):
                     break
             if step + 1 < max_new_tokens:
-                logits = self.forward(nxt[:, None], cache)[:, -1]
+                if self.fused:   # the launches `generate_graph` replays, issued one by one
+                    logits = self.step_fused(nxt[:, None], cache, slot)
+                    cache.filled += 1
+                else:
+                    logits = self.forward(nxt[:, None], cache)[:, -1]
         rows = out[:, :steps].tolist()
         if eos is not None:
             rows = [r[:r.index(eos) + 1] if eos in r else r for r in rows]

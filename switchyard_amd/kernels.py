@@ -103,6 +103,24 @@ def experts(h, idx, w, gate_up, down, mode="auto"):
     return E.combine(y, pos_of, idx, N)
 
 
+_ONE_EXPERT = {}
+
+
+def dense(x, weight):
+    """x [rows, K] @ weight [Nout, K]^T through the grouped kernels with a single expert that
+    owns every row: the weight-stream kernel up to 16 rows (one pass over the matrix), MFMA
+    tiles above. For the projections around the MoE layer at decode (q/k/v, output, lm_head),
+    which are weight streams like the experts are."""
+    rows = x.shape[0]
+    key = (rows, x.device)
+    if key not in _ONE_EXPERT:
+        _ONE_EXPERT[key] = torch.tensor([0, rows], dtype=torch.int32, device=x.device)
+    E = ext()
+    if rows <= 16 and weight.shape[1] <= 4096:
+        return E.grouped_gemv(x, None, weight[None], _ONE_EXPERT[key], rows, False, None, rows)
+    return E.grouped_gemm(x, None, weight[None], _ONE_EXPERT[key], None, 0, rows, False, None)
+
+
 # Up to this many tokens route and sort run as one launch of one workgroup (a decode step is
 # launch- and latency-bound in front of its two projections).
 FUSED_FRONT_MAX_TOKENS = 64

@@ -11,6 +11,7 @@ from switchyard_amd import _abi, kernels
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "switchyard_moe.h")
+DECODE_HEADER = os.path.join(ROOT, "include", "switchyard_decode.h")
 
 
 @pytest.fixture(scope="module")
@@ -18,13 +19,15 @@ def lib():
     return _abi.load_library()
 
 
-def declared_symbols():
-    text = open(HEADER).read()
+def declared_symbols(header=None):
+    text = open(header).read() if header else open(HEADER).read() + open(DECODE_HEADER).read()
     return re.findall(r"^SY_API\s+[\w\s\*]+?\b(sy_\w+)\(", text, flags=re.M)
 
 
 def test_header_declares_the_expected_entry_points():
-    assert sorted(declared_symbols()) == sorted(["sy_version", "sy_last_error", "sy_route", "sy_sort_workspace_bytes",
+    assert sorted(declared_symbols(DECODE_HEADER)) == ["sy_add_rmsnorm", "sy_decode_attention", "sy_qk_norm_rope_cache"]
+    assert sorted(os.listdir(os.path.join(ROOT, "include"))) == ["switchyard_decode.h", "switchyard_moe.h"]
+    assert sorted(declared_symbols(HEADER)) == sorted(["sy_version", "sy_last_error", "sy_route", "sy_sort_workspace_bytes",
                                                   "sy_sort_by_expert", "sy_route_sort",
                                                   "sy_grouped_gemv", "sy_grouped_gemm",
                                                   "sy_combine"])
@@ -43,6 +46,31 @@ def test_each_header_citation_names_a_reference_location():
     for name in ("sy_route", "sy_sort_by_expert", "sy_route_sort", "sy_grouped_gemv", "sy_grouped_gemm", "sy_combine"):
         comment = text[:text.index(f"SY_API int {name}(")].rsplit("/*", 1)[1]
         assert re.search(r"moe_kernels\.cu:\d+", comment), name
+
+
+def test_each_decode_citation_names_a_reference_location():
+    text = open(DECODE_HEADER).read()
+    for name in declared_symbols(DECODE_HEADER):
+        comment = text[:text.index(f"SY_API int {name}(")].rsplit("/*", 1)[1]
+        assert re.search(r"model\.py:\d+", comment), name
+
+
+def test_decode_argument_errors_and_empty_batches(lib):
+    assert lib.sy_add_rmsnorm(None, None, None, 1e-5, 4, 2052, None, None, None) == 1
+    assert b"multiple of 8" in lib.sy_last_error()
+    assert lib.sy_add_rmsnorm(None, None, None, 1e-5, 4, 16384, None, None, None) == 1
+    assert lib.sy_add_rmsnorm(None, None, None, 1e-5, 0, 2048, None, None, None) == 0
+    assert lib.sy_qk_norm_rope_cache(None, None, None, 1e-5, 0.0, None, None, 64, None, None, 2, 16, 5, 128, 64, None, None,
+                                     None, None) == 1
+    assert lib.sy_qk_norm_rope_cache(None, None, None, 1e-5, 0.0, None, None, 64, None, None, 2, 16, 16, 72, 64, None, None,
+                                     None, None) == 1
+    assert lib.sy_qk_norm_rope_cache(None, None, None, 1e-5, 0.0, None, None, 64, None, None, 0, 16, 16, 128, 64, None,
+                                     None, None, None) == 0
+    assert lib.sy_decode_attention(None, None, None, None, None, 2, 16, 16, 96, 64, None, None) == 1
+    assert b"64 or 128" in lib.sy_last_error()
+    assert lib.sy_decode_attention(None, None, None, None, None, 2, 16, 3, 128, 64, None, None) == 1
+    assert lib.sy_decode_attention(None, None, None, None, None, 0, 16, 16, 128, 64, None, None) == 0
+    assert lib.sy_decode_attention(None, None, None, None, None, 2, 16, 16, 128, 64, None, None) == 1  # null pointers
 
 
 def test_argument_errors_are_reported_without_a_device(lib):

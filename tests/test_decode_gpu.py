@@ -1,0 +1,198 @@
+"""The decode-step kernels around the MoE layer against the PyTorch operator sequences they
+replace (the reference's switchyard/model.py:14-17,61-84 with one new token per sequence).
+These are floating-point kernels: the check is a PyTorch reference of the same operation,
+in fp32 for attention and in fp16 (the reference's own arithmetic) for the norms and the
+rotary embedding, with the tolerance stated at each comparison."""
+
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from switchyard_amd import decoder as D
+from switchyard_amd import kernels
+
+pytestmark = pytest.mark.gpu
+
+ULP = 2.0 ** -10      # one unit in the last place of an fp16 value near 1
+
+
+def rnd(*shape, seed=0, std=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * std).half().cuda()
+
+
+@pytest.mark.parametrize("N,H", [(1, 2048), (8, 2048), (64, 2048), (5, 64), (3, 8192), (7, 520)])
+def test_add_rmsnorm(N, H):
+    x, d, w = rnd(N, H, seed=1), rnd(N, H, seed=2, std=0.3), 1 + rnd(H, seed=3, std=0.1)
+    E = kernels.ext()
+    # with a residual: the sum is the fp16 sum, bit for bit; the norm agrees to an fp16 rounding
+    # (the kernel's fp32 sum of squares runs in another order than torch's mean)
+    xo, h = E.add_rmsnorm(x, d, w, 1e-5)
+    assert torch.equal(xo, x + d)
+    want = D._rms(x + d, w, 1e-5)
+    assert torch.allclose(h.float(), want.float(), rtol=2 * ULP, atol=1e-4)
+    assert (h != want).float().mean().item() < 0.01
+    # without: x is passed through untouched; in place: x itself is updated
+    same, h0 = E.add_rmsnorm(x, None, w, 1e-5)
+    assert same is x and torch.allclose(h0.float(), D._rms(x, w, 1e-5).float(), rtol=2 * ULP, atol=1e-4)
+    x2 = x.clone()
+    xo2, h2 = E.add_rmsnorm(x2, d, w, 1e-5, x_out=x2)
+    assert xo2 is x2 and torch.equal(x2, xo) and torch.equal(h2, h)
+
+
+def torch_qk_step(qkv, L, s, cos, sin, positions, clip):
+    """q, k (normed, clamped, rotated) and v of one new token, as Decoder.step_static does."""
+    B = qkv.shape[0]
+    qd, kvd = s.heads * s.head_dim, s.kv_heads * s.head_dim
+    q = D._rms(qkv[:, :qd], L["q_norm"], s.rms_eps)
+    k = D._rms(qkv[:, qd:qd + kvd], L["k_norm"], s.rms_eps)
+    v = qkv[:, qd + kvd:]
+    if clip:
+        q, k, v = q.clamp(-clip, clip), k.clamp(-clip, clip), v.clamp(-clip, clip)
+    q = q.view(B, s.heads, 1, s.head_dim)
+    k = k.view(B, s.kv_heads, 1, s.head_dim)
+    c, sn = cos[positions][:, None, None], sin[positions][:, None, None]
+    return D._rotate(q, c, sn), D._rotate(k, c, sn), v.reshape(B, s.kv_heads, 1, s.head_dim)
+
+
+@pytest.mark.parametrize("B,heads,kv_heads,hd,clip", [(8, 16, 16, 128, None), (3, 8, 2, 64, None), (64, 16, 16, 128, 0.4),
+                                                     (1, 4, 4, 64, None), (5, 32, 8, 128, 1.5)])
+def test_qk_norm_rope_cache(B, heads, kv_heads, hd, clip):
+    s = D.Shape(hidden=512, heads=heads, kv_heads=kv_heads, head_dim=hd, clip_qkv=clip)
+    cap, max_pos, slot_at = 37, 96, 11
+    dec = D.Decoder(s, {"embed": torch.zeros(1, 8, dtype=torch.float16, device="cuda"), "layers": []}, moe=lambda i, h: h,
+                    max_positions=max_pos, attention="torch")
+    qd, kvd = heads * hd, kv_heads * hd
+    qkv = rnd(B, qd + 2 * kvd, seed=4, std=0.7)
+    L = {"q_norm": 1 + rnd(qd, seed=5, std=0.1), "k_norm": 1 + rnd(kvd, seed=6, std=0.1)}
+    positions = torch.randint(0, max_pos, (B,), generator=torch.Generator().manual_seed(7)).cuda()
+    slot = torch.tensor([slot_at], device="cuda")
+    kc, vc = rnd(B, kv_heads, cap, hd, seed=8), rnd(B, kv_heads, cap, hd, seed=9)
+    kc0, vc0 = kc.clone(), vc.clone()
+    q = kernels.ext().qk_norm_rope_cache(qkv, L["q_norm"], L["k_norm"], s.rms_eps, clip, dec.cos, dec.sin, positions, slot,
+                                         heads, kv_heads, hd, kc, vc)
+    wq, wk, wv = torch_qk_step(qkv, L, s, dec.cos, dec.sin, positions, clip)
+    # one fp16 rounding of the norm can differ (order of the fp32 sum of squares); it passes
+    # through one rotary product, so two roundings of a value of the tensor's size
+    tol = dict(rtol=4 * ULP, atol=4 * ULP)
+    assert torch.allclose(q.float(), wq.reshape(B, qd).float(), **tol)
+    assert torch.allclose(kc[:, :, slot_at].float(), wk[:, :, 0].float(), **tol)
+    assert torch.equal(vc[:, :, slot_at], wv[:, :, 0])
+    assert (q != wq.reshape(B, qd)).float().mean().item() < 0.02
+    keep = torch.ones(cap, dtype=torch.bool, device="cuda")
+    keep[slot_at] = False
+    assert torch.equal(kc[:, :, keep], kc0[:, :, keep]) and torch.equal(vc[:, :, keep], vc0[:, :, keep])
+    # a slot outside the cache writes nothing
+    kernels.ext().qk_norm_rope_cache(qkv, L["q_norm"], L["k_norm"], s.rms_eps, clip, dec.cos, dec.sin, positions,
+                                     torch.tensor([cap], device="cuda"), heads, kv_heads, hd, kc, vc)
+    assert torch.equal(kc[:, :, keep], kc0[:, :, keep]) and torch.equal(vc[:, :, keep], vc0[:, :, keep])
+
+
+@pytest.mark.parametrize("B,heads,kv_heads,hd,cap,slot_at", [
+    (8, 16, 16, 128, 640, 600),    # OLMoE at batch 8: 16 wavefronts per (sequence, head)
+    (64, 16, 16, 128, 200, 199),   # many pairs: 4 wavefronts each; the last slot of the cache
+    (3, 8, 2, 64, 77, 50),         # grouped-query heads, head_dim 64, ragged sizes
+    (2, 4, 4, 128, 9, 0),          # a single visible key
+    (2, 4, 1, 64, 33, 2),
+    (40, 16, 4, 64, 130, 129),
+])
+def test_decode_attention(B, heads, kv_heads, hd, cap, slot_at):
+    g = torch.Generator().manual_seed(11)
+    q = rnd(B, heads * hd, seed=12, std=1.5)
+    kc, vc = rnd(B, kv_heads, cap, hd, seed=13), rnd(B, kv_heads, cap, hd, seed=14)
+    # left padding of different lengths, plus holes: any pattern of real positions must work
+    real = torch.rand(B, cap, generator=g) > 0.2
+    pad = torch.randint(0, max(1, slot_at), (B,), generator=g)
+    real &= torch.arange(cap)[None] >= pad[:, None]
+    real[:, slot_at] = True
+    real = real.cuda()
+    slot = torch.tensor([slot_at], device="cuda")
+    out = kernels.ext().decode_attention(q, kc, vc, real, slot, heads)
+    mask = (real & (torch.arange(cap, device="cuda")[None] <= slot_at))[:, None, None, :]
+    want = F.scaled_dot_product_attention(q.view(B, heads, 1, hd).float(), kc.float(), vc.float(), attn_mask=mask,
+                                          enable_gqa=heads != kv_heads)
+    # fp32 inside, one rounding to fp16 at the end
+    assert torch.allclose(out.float(), want.reshape(B, heads * hd), rtol=2 * ULP, atol=1e-3)
+
+
+def test_decode_attention_without_a_real_key_gives_zeros():
+    B, heads, hd, cap = 2, 4, 64, 16
+    q, kc, vc = rnd(B, heads * hd), rnd(B, heads, cap, hd), rnd(B, heads, cap, hd)
+    real = torch.zeros(B, cap, dtype=torch.bool, device="cuda")
+    real[1, 3] = True
+    out = kernels.ext().decode_attention(q, kc, vc, real, torch.tensor([5], device="cuda"), heads)
+    assert torch.equal(out[0], torch.zeros_like(out[0]))
+    assert torch.allclose(out[1].view(heads, hd).float(), vc[1, :, 3].float(), atol=1e-3)
+
+
+@pytest.mark.parametrize("rows,Nout,K", [(1, 6144, 2048), (8, 6144, 2048), (8, 2048, 2048), (16, 2048, 2048), (8, 50304, 2048),
+                                        (8, 1000, 512), (3, 1001, 512), (17, 2048, 2048), (64, 6144, 2048),
+                                        (64, 50304, 2048), (40, 1000, 512)])
+def test_dense_projection(rows, Nout, K):
+    """A projection as a single-expert call of the grouped kernels: fp32 accumulation, one
+    rounding to fp16, compared with the fp32 product."""
+    x, w = rnd(rows, K, seed=20), rnd(Nout, K, seed=21, std=0.03)
+    got = kernels.dense(x, w)
+    want = x.float() @ w.float().T
+    assert got.shape == (rows, Nout)
+    assert torch.allclose(got.float(), want, rtol=2 * ULP, atol=2e-3)
+
+
+def model(seed, batch, **kw):
+    s = D.Shape(**{**dict(vocab=1000, hidden=512, intermediate=256, layers=3, heads=8, kv_heads=8, head_dim=64, experts=64,
+                          top_k=8), **kw})
+    w = D.random_weights(s, device="cuda", seed=seed, std=0.05)
+    ps = [torch.randint(3, s.vocab, (10 + 4 * b,), generator=torch.Generator().manual_seed(b)).tolist()
+          for b in range(batch)]
+    return s, w, ps
+
+
+@pytest.mark.parametrize("kw", [{}, {"kv_heads": 2}, {"head_dim": 128, "heads": 4, "kv_heads": 4}, {"clip_qkv": 0.5},
+                                {"norm_topk_prob": True}])
+def test_a_step_on_the_decode_kernels_gives_the_logits_of_the_torch_step(kw):
+    """Same weights, same prefilled cache, one new token per sequence of a left-padded batch:
+    `step_fused` against `step_static` (PyTorch attention, the same MoE hook). Tolerance 2e-2
+    on the logits, as for the MoE layer; the caches agree to fp16 roundings."""
+    s, w, ps = model(3, 6, **kw)
+    fused = D.Decoder(s, w, max_positions=128, attention="kernels")
+    plain = D.Decoder(s, w, max_positions=128, attention="torch")
+    assert fused.fused and not plain.fused
+    B, P = len(ps), max(len(p) for p in ps)
+    tokens = torch.zeros(B, P, dtype=torch.long)
+    valid = torch.zeros(B, P, dtype=torch.bool)
+    for b, p in enumerate(ps):
+        tokens[b, P - len(p):] = torch.tensor(p)
+        valid[b, P - len(p):] = True
+    tokens, valid = tokens.cuda(), valid.cuda()
+    feed = torch.randint(3, s.vocab, (3, B, 1), generator=torch.Generator().manual_seed(9)).cuda()
+    caches, logits = [], []
+    for m in (fused, plain):
+        cache = D.KVCache(s, B, P + 4, torch.float16, "cuda")
+        m.forward(tokens, cache, valid)
+        slot = torch.tensor([cache.filled], device="cuda")
+        keys = torch.arange(cache.capacity, device="cuda")
+        logits.append(torch.stack([m.step(tok, cache, slot, keys) for tok in feed]))
+        caches.append(cache)
+    assert int(caches[0].next_position[0]) == int(caches[1].next_position[0]) == len(ps[0]) + 3
+    assert (logits[0].float() - logits[1].float()).abs().max().item() < 2e-2
+    assert torch.equal(caches[0].real, caches[1].real)
+    assert (caches[0].k.float() - caches[1].k.float()).abs().max().item() < 2e-2
+    assert (caches[0].v.float() - caches[1].v.float()).abs().max().item() < 2e-2
+
+
+def test_generation_on_the_decode_kernels_picks_the_torch_models_tokens_up_to_ties():
+    """Greedy decoding through `step_fused`; every picked token is the PyTorch-attention
+    model's top-1 for the same prefix, or within the logits tolerance of it."""
+    s, w, ps = model(5, 4)
+    fused = D.Decoder(s, w, max_positions=128, attention="kernels")
+    plain = D.Decoder(s, w, max_positions=128, attention="torch")
+    picked = fused.generate(ps, 12)
+    assert fused.generate_graph(ps, 12) == picked
+    tol = 2e-2
+    for prompt, out in zip(ps, picked):
+        seq = torch.tensor([prompt + out], device="cuda")
+        lg = plain.forward(seq)[0, len(prompt) - 1:len(prompt) - 1 + len(out)].float()
+        chosen = lg.gather(1, torch.tensor(out, device="cuda")[:, None])[:, 0]
+        assert (lg.max(-1).values - chosen).max().item() <= 2 * tol
