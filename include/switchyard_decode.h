@@ -27,6 +27,23 @@ extern "C" {
 SY_API int sy_add_rmsnorm(const void* x, const void* delta, const void* weight, float eps, int N, int H, void* x_out,
                           void* h_out, void* stream);
 
+/* sy_add_rmsnorm that also takes the router's logits of the normalised rows, so that the router
+ * GEMM of the MoE layer (`F.linear(h, router)`, switchyard/kernels.py:30-32 after
+ * switchyard/model.py:121) needs no launch of its own at decode.
+ * router f16 [E,H] -> logits f16 [N,E] = f16(h_out @ router^T), fp32 sums; the other arguments
+ * and results as sy_add_rmsnorm. Limits: as sy_add_rmsnorm, 1 <= E <= 1024. */
+SY_API int sy_add_rmsnorm_logits(const void* x, const void* delta, const void* weight, float eps, const void* router,
+                                 int E, int N, int H, void* x_out, void* h_out, void* logits, void* stream);
+
+/* sy_combine folded into the residual add and the next RMS norm: replaces combine()
+ * (switchyard/csrc/moe_kernels.cu:435-444) followed by `x = x + moe(i, h)` and the rmsnorm of
+ * the next block (switchyard/model.py:142,119 or :130).
+ * y f16 [M,H], pos_of int32 [N*k], idx int32 [N,k] as sy_combine takes them; x f16 [N,H] ->
+ * x_out = f16(x + d) with d the f16 result sy_combine would give (the same bits), and
+ * h_out = the RMS norm of x_out as sy_add_rmsnorm. Limits: as sy_add_rmsnorm, 1 <= k <= 64. */
+SY_API int sy_combine_add_rmsnorm(const void* y, const int32_t* pos_of, const int32_t* idx, int k, const void* x,
+                                  const void* weight, float eps, int N, int H, void* x_out, void* h_out, void* stream);
+
 /* What follows the q/k/v projections of one new token per sequence; replaces the rmsnorm of q
  * and k, the clamp, the rotary embedding and the cache write of _attention()
  * (switchyard/model.py:64-77) with T = 1.

@@ -36,6 +36,10 @@ SIGNATURES = {
     "sy_combine": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p]),
     "sy_add_rmsnorm": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_int, _c_int, _c_void_p, _c_void_p,
                                 _c_void_p]),
+    "sy_add_rmsnorm_logits": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_int, _c_int,
+                                       _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
+    "sy_combine_add_rmsnorm": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_float, _c_int,
+                                        _c_int, _c_void_p, _c_void_p, _c_void_p]),
     "sy_qk_norm_rope_cache": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_float, _c_void_p, _c_void_p, _c_int,
                                        _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p,
                                        _c_void_p, _c_void_p, _c_void_p]),
@@ -182,9 +186,10 @@ class Ext:
         return out
 
     # ---- the decode-step kernels around the MoE layer (include/switchyard_decode.h)
-    def add_rmsnorm(self, x, delta, weight, eps, x_out=None):
+    def add_rmsnorm(self, x, delta, weight, eps, x_out=None, router=None):
         """x [N, H] (+ delta [N, H] or None) -> (x + delta, weight * rmsnorm(x + delta)).
-        With delta None the first result is x itself; x_out may be x for an update in place."""
+        With delta None the first result is x itself; x_out may be x for an update in place.
+        With `router` [E, H] a third result is the logits [N, E] of the normalised rows."""
         _check(x, "x", torch.float16)
         _check(weight, "weight", torch.float16)
         N, H = x.shape
@@ -200,10 +205,40 @@ class Ext:
             if x_out.shape != x.shape:
                 raise RuntimeError("add_rmsnorm: x_out must have x's shape")
         h = torch.empty_like(x)
-        self._call(self.lib.sy_add_rmsnorm, x.data_ptr(), delta.data_ptr() if delta is not None else None,
-                   weight.data_ptr(), float(eps), N, H, x_out.data_ptr() if delta is not None else None, h.data_ptr(),
-                   _stream())
-        return (x_out if delta is not None else x), h
+        d_ptr = delta.data_ptr() if delta is not None else None
+        o_ptr = x_out.data_ptr() if delta is not None else None
+        first = x_out if delta is not None else x
+        if router is None:
+            self._call(self.lib.sy_add_rmsnorm, x.data_ptr(), d_ptr, weight.data_ptr(), float(eps), N, H, o_ptr,
+                       h.data_ptr(), _stream())
+            return first, h
+        _check(router, "router", torch.float16)
+        if router.dim() != 2 or router.shape[1] != H:
+            raise RuntimeError("add_rmsnorm: router must be [E, H]")
+        logits = torch.empty((N, router.shape[0]), dtype=torch.float16, device=x.device)
+        self._call(self.lib.sy_add_rmsnorm_logits, x.data_ptr(), d_ptr, weight.data_ptr(), float(eps), router.data_ptr(),
+                   router.shape[0], N, H, o_ptr, h.data_ptr(), logits.data_ptr(), _stream())
+        return first, h, logits
+
+    def combine_add_rmsnorm(self, y, pos_of, idx, x, weight, eps, x_out=None):
+        """combine(y, pos_of, idx) added to x [N, H] and normalised in one launch ->
+        (x + combine, weight * rmsnorm(x + combine)); x_out may be x."""
+        _check(y, "y", torch.float16)
+        _check(pos_of, "pos_of", torch.int32)
+        _check(idx, "idx", torch.int32)
+        _check(x, "x", torch.float16)
+        _check(weight, "weight", torch.float16)
+        N, H = x.shape
+        k = idx.shape[1]
+        if y.shape[1] != H or weight.numel() != H or pos_of.numel() < N * k or idx.shape[0] < N:
+            raise RuntimeError("combine_add_rmsnorm: shapes of y / pos_of / idx / weight do not match x")
+        if x_out is None:
+            x_out = torch.empty_like(x)
+        _check(x_out, "x_out", torch.float16)
+        h = torch.empty_like(x)
+        self._call(self.lib.sy_combine_add_rmsnorm, y.data_ptr(), pos_of.data_ptr(), idx.data_ptr(), k, x.data_ptr(),
+                   weight.data_ptr(), float(eps), N, H, x_out.data_ptr(), h.data_ptr(), _stream())
+        return x_out, h
 
     def qk_norm_rope_cache(self, qkv, q_norm, k_norm, eps, clip, cos, sin, positions, slot, heads, kv_heads, head_dim,
                            kcache, vcache):

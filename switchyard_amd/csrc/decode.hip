@@ -6,7 +6,10 @@
 // KV cache it has to read. Three kernels replace them (the projections themselves go through
 // the weight-stream kernel with a single "expert"):
 //
-//   add_rmsnorm           x += delta; h = w * f16(x * rsqrt(mean(x^2) + eps))       (one row per workgroup)
+//   add_rmsnorm           x += delta; h = w * f16(x * rsqrt(mean(x^2) + eps)), one row per workgroup;
+//                         delta may be the combine of the MoE layer's rows (combine_add_rmsnorm),
+//                         and the router's logits of h may come out of the same launch
+//                         (add_rmsnorm_logits)
 //   qk_norm_rope_cache    q/k RMS norm over the whole projection, clamp, rotary embedding, and
 //                         the new key and value written into the cache at `slot`
 //   decode_attention      one query per (sequence, head) against the cache: a single pass over
@@ -36,20 +39,57 @@ __device__ __forceinline__ float block_sum(float v, float* lds, int slot_base) {
   return lds[slot_base] + lds[slot_base + 1] + lds[slot_base + 2] + lds[slot_base + 3];
 }
 
+constexpr int ROW_MAX_K = 64;  // choices per token the combining variant ranks in one wavefront
+
+// One workgroup per token (row). The residual `delta` is either a tensor, or (COMBINE) the
+// token's k expert outputs summed in fp32 in ascending expert id and rounded to f16 once,
+// exactly as the combine kernel leaves it; then x_out = f16(x + delta) and h = the RMS norm
+// of x_out. With LOGITS the normalised row stays in LDS and the four wavefronts also take its
+// dot products with the E rows of the router (fp32 sums, one rounding to f16), so that the
+// router needs no launch of its own.
+template <bool COMBINE, bool LOGITS>
 __global__ void __launch_bounds__(ROW_THREADS)
-add_rmsnorm_kernel(const half_t* x, const half_t* __restrict__ delta, const half_t* __restrict__ weight, float eps,
-                   int H, half_t* x_out, half_t* __restrict__ h_out) {  // x_out may be x
+row_kernel(const half_t* x, const half_t* __restrict__ delta, const half_t* __restrict__ y,
+           const int* __restrict__ pos_of, const int* __restrict__ idx, int k, const half_t* __restrict__ weight,
+           float eps, const half_t* __restrict__ router, int E, int H, half_t* x_out, half_t* __restrict__ h_out,
+           half_t* __restrict__ logits) {  // x_out may be x
+  extern __shared__ __attribute__((aligned(16))) half_t hs[];  // LOGITS: the normalised row [H]
   __shared__ float part[4];
-  const size_t row = (size_t)blockIdx.x * H;
+  __shared__ int rows[ROW_MAX_K];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const size_t row = (size_t)t * H;
   const int chunks = H >> 3;
+  if (COMBINE) {
+    // rank the k choices by (expert id, slot); rows[] lists their rows of y in that order
+    if (tid < WAVE) {
+      const int mine = tid < k ? idx[(size_t)t * k + tid] : 0x7fffffff;
+      const int src = tid < k ? pos_of[(size_t)t * k + tid] : 0;
+      int rank = 0;
+      for (int j = 0; j < k; ++j) {
+        const int other = read_lane(mine, j);
+        rank += (other < mine) || (other == mine && j < tid);
+      }
+      if (tid < k) rows[rank] = src;
+    }
+    __syncthreads();
+  }
   half8_t v[MAX_CHUNKS];
   float ss = 0.f;
 #pragma unroll
   for (int i = 0; i < MAX_CHUNKS; ++i) {
-    const int c = threadIdx.x + i * ROW_THREADS;
+    const int c = tid + i * ROW_THREADS;
     if (c < chunks) {
       v[i] = *reinterpret_cast<const half8_t*>(x + row + c * 8);
-      if (delta) {
+      if (COMBINE) {
+        float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < k; ++j) {
+          const half8_t e = *reinterpret_cast<const half8_t*>(y + (size_t)rows[j] * H + c * 8);
+#pragma unroll
+          for (int q = 0; q < 8; ++q) acc[q] += (float)e[q];
+        }
+#pragma unroll
+        for (int q = 0; q < 8; ++q) v[i][q] = (half_t)((float)v[i][q] + (float)(half_t)acc[q]);
+      } else if (delta) {
         const half8_t d = *reinterpret_cast<const half8_t*>(delta + row + c * 8);
 #pragma unroll
         for (int j = 0; j < 8; ++j) v[i][j] = (half_t)((float)v[i][j] + (float)d[j]);
@@ -61,7 +101,7 @@ add_rmsnorm_kernel(const half_t* x, const half_t* __restrict__ delta, const half
   const float rs = rsqrtf(block_sum(ss, part, 0) / (float)H + eps);
 #pragma unroll
   for (int i = 0; i < MAX_CHUNKS; ++i) {
-    const int c = threadIdx.x + i * ROW_THREADS;
+    const int c = tid + i * ROW_THREADS;
     if (c < chunks) {
       const half8_t w = *reinterpret_cast<const half8_t*>(weight + c * 8);
       half8_t h;
@@ -69,6 +109,33 @@ add_rmsnorm_kernel(const half_t* x, const half_t* __restrict__ delta, const half
       for (int j = 0; j < 8; ++j) h[j] = (half_t)((float)w[j] * (float)(half_t)((float)v[i][j] * rs));
       if (x_out) *reinterpret_cast<half8_t*>(x_out + row + c * 8) = v[i];
       *reinterpret_cast<half8_t*>(h_out + row + c * 8) = h;
+      if (LOGITS) *reinterpret_cast<half8_t*>(hs + c * 8) = h;
+    }
+  }
+  if (!LOGITS) return;
+  __syncthreads();
+  // wavefront w takes experts w, w + 4, ...: four at a time, so that 4 loads per lane are in flight
+  const int wave = tid >> 6, lane = tid & 63;
+  for (int e0 = wave; e0 < E; e0 += 16) {
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int c = lane; c < chunks; c += WAVE) {
+      const half8_t hv = *reinterpret_cast<const half8_t*>(hs + c * 8);
+      half8_t r[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int e = e0 + 4 * u;
+        r[u] = *reinterpret_cast<const half8_t*>(router + (size_t)(e < E ? e : e0) * H + c * 8);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[u] += (float)hv[j] * (float)r[u][j];
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const float total = wave_sum(acc[u]);
+      const int e = e0 + 4 * u;
+      if (lane == 0 && e < E) logits[(size_t)t * E + e] = (half_t)total;
     }
   }
 }
@@ -309,16 +376,45 @@ __global__ void decode_attention_kernel(const half_t* __restrict__ q, const half
 
 }  // namespace
 
+#define ROW_LIMITS(what)                                                                          \
+  SY_REQUIRE(N >= 0 && H >= 8 && H % 8 == 0 && H <= 8 * ROW_THREADS * MAX_CHUNKS,                \
+             what ": N = %d, H = %d (a multiple of 8 up to %d)", N, H, 8 * ROW_THREADS * MAX_CHUNKS)
+
 extern "C" SY_API int sy_add_rmsnorm(const void* x, const void* delta, const void* weight, float eps, int N, int H,
                                      void* x_out, void* h_out, void* stream) {
-  SY_REQUIRE(N >= 0 && H >= 8 && H % 8 == 0 && H <= 8 * ROW_THREADS * MAX_CHUNKS,
-             "add_rmsnorm: N = %d, H = %d (a multiple of 8 up to %d)", N, H, 8 * ROW_THREADS * MAX_CHUNKS);
+  ROW_LIMITS("add_rmsnorm");
   if (N == 0) return SY_OK;
   SY_REQUIRE(x && weight && h_out, "add_rmsnorm: null pointer");
-  add_rmsnorm_kernel<<<N, ROW_THREADS, 0, (hipStream_t)stream>>>((const half_t*)x, (const half_t*)delta,
-                                                                 (const half_t*)weight, eps, H, (half_t*)x_out,
-                                                                 (half_t*)h_out);
+  row_kernel<false, false><<<N, ROW_THREADS, 0, (hipStream_t)stream>>>(
+      (const half_t*)x, (const half_t*)delta, nullptr, nullptr, nullptr, 0, (const half_t*)weight, eps, nullptr, 0, H,
+      (half_t*)x_out, (half_t*)h_out, nullptr);
   return sy_check_launch("add_rmsnorm");
+}
+
+extern "C" SY_API int sy_add_rmsnorm_logits(const void* x, const void* delta, const void* weight, float eps,
+                                            const void* router, int E, int N, int H, void* x_out, void* h_out,
+                                            void* logits, void* stream) {
+  ROW_LIMITS("add_rmsnorm_logits");
+  SY_REQUIRE(E >= 1 && E <= 1024, "add_rmsnorm_logits: 1 <= E <= 1024 (got %d)", E);
+  if (N == 0) return SY_OK;
+  SY_REQUIRE(x && weight && h_out && router && logits, "add_rmsnorm_logits: null pointer");
+  row_kernel<false, true><<<N, ROW_THREADS, (size_t)H * sizeof(half_t), (hipStream_t)stream>>>(
+      (const half_t*)x, (const half_t*)delta, nullptr, nullptr, nullptr, 0, (const half_t*)weight, eps,
+      (const half_t*)router, E, H, (half_t*)x_out, (half_t*)h_out, (half_t*)logits);
+  return sy_check_launch("add_rmsnorm_logits");
+}
+
+extern "C" SY_API int sy_combine_add_rmsnorm(const void* y, const int32_t* pos_of, const int32_t* idx, int k, const void* x,
+                                             const void* weight, float eps, int N, int H, void* x_out, void* h_out,
+                                             void* stream) {
+  ROW_LIMITS("combine_add_rmsnorm");
+  SY_REQUIRE(k >= 1 && k <= ROW_MAX_K, "combine_add_rmsnorm: 1 <= k <= %d (got %d)", ROW_MAX_K, k);
+  if (N == 0) return SY_OK;
+  SY_REQUIRE(y && pos_of && idx && x && weight && h_out, "combine_add_rmsnorm: null pointer");
+  row_kernel<true, false><<<N, ROW_THREADS, 0, (hipStream_t)stream>>>(
+      (const half_t*)x, nullptr, (const half_t*)y, pos_of, idx, k, (const half_t*)weight, eps, nullptr, 0, H,
+      (half_t*)x_out, (half_t*)h_out, nullptr);
+  return sy_check_launch("combine_add_rmsnorm");
 }
 
 extern "C" SY_API int sy_qk_norm_rope_cache(const void* qkv, const void* q_norm, const void* k_norm, float eps, float clip,

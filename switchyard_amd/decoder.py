@@ -132,6 +132,7 @@ class Decoder:
         kernels where they apply (GPU, fp16, head_dim 64 or 128)."""
         self.s, self.w = shape, weights
         self.moe = moe or self.kernel_moe
+        self._own_moe = moe is None     # the step may then fold the layer's ends into its neighbours
         dev = weights["embed"].device
         can = (dev.type == "cuda" and weights["embed"].dtype == torch.float16 and shape.head_dim in (64, 128)
                and shape.hidden % 8 == 0 and shape.hidden <= 8192 and shape.heads * shape.head_dim <= 8192)
@@ -269,17 +270,23 @@ class Decoder:
         positions = cache.next_position
         cache.real.index_fill_(1, slot, True)
         x = F.embedding(tok[:, 0], W["embed"])
-        delta = None
+        x, xn = E.add_rmsnorm(x, None, W["layers"][0]["attn_norm"], s.rms_eps)
         for i in range(s.layers):
             L = W["layers"][i]
-            x, xn = E.add_rmsnorm(x, delta, L["attn_norm"], s.rms_eps, x_out=x)
+            after = W["layers"][i + 1]["attn_norm"] if i + 1 < s.layers else W["final_norm"]
             q = E.qk_norm_rope_cache(kernels.dense(xn, wqkv[i]), L["q_norm"], L["k_norm"], s.rms_eps, s.clip_qkv,
                                      self.cos, self.sin, positions, slot, s.heads, s.kv_heads, s.head_dim,
                                      cache.k[i], cache.v[i])
             a = E.decode_attention(q, cache.k[i], cache.v[i], cache.real, slot, s.heads)
-            x, h = E.add_rmsnorm(x, kernels.dense(a, L["wo"]), L["mlp_norm"], s.rms_eps, x_out=x)
-            delta = self.moe(i, h)
-        x, xn = E.add_rmsnorm(x, delta, W["final_norm"], s.rms_eps, x_out=x)
+            o = kernels.dense(a, L["wo"])
+            if self._own_moe and s.experts <= 1024 and s.top_k <= 64:
+                # the router's logits come out of the norm's launch, and combine goes into the next norm's
+                x, h, logits = E.add_rmsnorm(x, o, L["mlp_norm"], s.rms_eps, x_out=x, router=L["router"])
+                y, pos_of, idx = kernels.experts_rows(h, logits, L["gate_up"], L["down"], s.top_k, s.norm_topk_prob)
+                x, xn = E.combine_add_rmsnorm(y, pos_of, idx, x, after, s.rms_eps, x_out=x)
+            else:
+                x, h = E.add_rmsnorm(x, o, L["mlp_norm"], s.rms_eps, x_out=x)
+                x, xn = E.add_rmsnorm(x, self.moe(i, h), after, s.rms_eps, x_out=x)
         cache.next_position += 1
         slot += 1
         return kernels.dense(xn, W["lm_head"])

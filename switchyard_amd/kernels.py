@@ -107,34 +107,50 @@ _ONE_EXPERT = {}
 
 
 def dense(x, weight):
-    """x [rows, K] @ weight [Nout, K]^T through the grouped kernels with a single expert that
-    owns every row: the weight-stream kernel up to 16 rows (one pass over the matrix), MFMA
-    tiles above. For the projections around the MoE layer at decode (q/k/v, output, lm_head),
-    which are weight streams like the experts are."""
+    """x [rows, K] @ weight [Nout, K]^T for the projections around the MoE layer at decode
+    (q/k/v, output, lm_head), which are weight streams like the experts are. Up to 16 rows the
+    weight-stream kernel runs with a single expert that owns every row (one pass over the
+    matrix; measured in a replayed graph at 8 rows: 9.7 us for [6144, 2048], 6.8 us for
+    [2048, 2048], 36.9 us for [50304, 2048], against 12.4, 8.8 and 52.9 us for the library
+    GEMM). Above that a plain GEMM is the library's job (12.5 us at 64 rows where the kernel's
+    four passes take 33.6 us)."""
     rows = x.shape[0]
+    if rows > 16 or weight.shape[1] > 4096 or weight.shape[1] % 8:
+        return F.linear(x, weight)
     key = (rows, x.device)
     if key not in _ONE_EXPERT:
         _ONE_EXPERT[key] = torch.tensor([0, rows], dtype=torch.int32, device=x.device)
-    E = ext()
-    if rows <= 16 and weight.shape[1] <= 4096:
-        return E.grouped_gemv(x, None, weight[None], _ONE_EXPERT[key], rows, False, None, rows)
-    return E.grouped_gemm(x, None, weight[None], _ONE_EXPERT[key], None, 0, rows, False, None)
+    return ext().grouped_gemv(x, None, weight[None], _ONE_EXPERT[key], rows, False, None, rows)
 
 
 # Up to this many tokens route and sort run as one launch of one workgroup (a decode step is
-# launch- and latency-bound in front of its two projections).
-FUSED_FRONT_MAX_TOKENS = 64
+# launch- and latency-bound in front of its two projections). Measured in a replayed graph, one
+# launch against route + sort_by_expert: 8 tokens 3.7 against 6.5 us, 16 tokens 6.5 against 6.6,
+# 32 tokens 9.2 against 6.8, 64 tokens 14.6 against 6.9 (one compute unit routes every token).
+FUSED_FRONT_MAX_TOKENS = 16
+
+
+def experts_rows(h, logits, gate_up, down, top_k, norm_topk_prob, mode="auto"):
+    """The MoE layer from its router logits [N, E] up to, not including, combine: returns
+    (y [N*k, H] expert outputs scaled by the router weights, pos_of, idx), which `combine`
+    or a kernel that folds it into what follows takes. Route and sort are one launch up to
+    FUSED_FRONT_MAX_TOKENS tokens."""
+    E = ext()
+    N, n_experts = h.shape[0], gate_up.shape[0]
+    if 0 < N <= FUSED_FRONT_MAX_TOKENS and n_experts <= 128 and top_k <= 8 and logits.dtype == torch.float16:
+        idx, w, counts, offsets, token, wsorted, pos_of = E.route_sort(logits, top_k, norm_topk_prob)
+    else:
+        idx, w = E.route(logits, top_k, norm_topk_prob)
+        counts, offsets, token, wsorted, pos_of = E.sort_by_expert(idx, w, n_experts)
+    if mode == "auto":
+        mode = _auto(N, idx.numel(), n_experts)
+    return ffn(h, token, offsets, counts, wsorted, gate_up, down, idx.numel(), mode), pos_of, idx
 
 
 def moe_layer(h, router, gate_up, down, top_k, norm_topk_prob, mode="auto"):
     N, n_experts = h.shape[0], gate_up.shape[0]
     if 0 < N <= FUSED_FRONT_MAX_TOKENS and n_experts <= 128 and top_k <= 8 and h.dtype == torch.float16:
-        E = ext()
-        idx, w, counts, offsets, token, wsorted, pos_of = E.route_sort(F.linear(h, router).contiguous(), top_k,
-                                                                       norm_topk_prob)
-        if mode == "auto":
-            mode = _auto(N, idx.numel(), n_experts)
-        y = ffn(h, token, offsets, counts, wsorted, gate_up, down, idx.numel(), mode)
-        return E.combine(y, pos_of, idx, N)
+        y, pos_of, idx = experts_rows(h, F.linear(h, router).contiguous(), gate_up, down, top_k, norm_topk_prob, mode)
+        return ext().combine(y, pos_of, idx, N)
     idx, w = route(h, router, top_k, norm_topk_prob)
     return experts(h, idx, w, gate_up, down, mode)

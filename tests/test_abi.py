@@ -25,7 +25,8 @@ def declared_symbols(header=None):
 
 
 def test_header_declares_the_expected_entry_points():
-    assert sorted(declared_symbols(DECODE_HEADER)) == ["sy_add_rmsnorm", "sy_decode_attention", "sy_qk_norm_rope_cache"]
+    assert sorted(declared_symbols(DECODE_HEADER)) == ["sy_add_rmsnorm", "sy_add_rmsnorm_logits", "sy_combine_add_rmsnorm",
+                                                       "sy_decode_attention", "sy_qk_norm_rope_cache"]
     assert sorted(os.listdir(os.path.join(ROOT, "include"))) == ["switchyard_decode.h", "switchyard_moe.h"]
     assert sorted(declared_symbols(HEADER)) == sorted(["sy_version", "sy_last_error", "sy_route", "sy_sort_workspace_bytes",
                                                   "sy_sort_by_expert", "sy_route_sort",
@@ -52,7 +53,7 @@ def test_each_decode_citation_names_a_reference_location():
     text = open(DECODE_HEADER).read()
     for name in declared_symbols(DECODE_HEADER):
         comment = text[:text.index(f"SY_API int {name}(")].rsplit("/*", 1)[1]
-        assert re.search(r"model\.py:\d+", comment), name
+        assert re.search(r"(model|kernels)\.py:\d+", comment), name
 
 
 def test_decode_argument_errors_and_empty_batches(lib):
@@ -60,6 +61,11 @@ def test_decode_argument_errors_and_empty_batches(lib):
     assert b"multiple of 8" in lib.sy_last_error()
     assert lib.sy_add_rmsnorm(None, None, None, 1e-5, 4, 16384, None, None, None) == 1
     assert lib.sy_add_rmsnorm(None, None, None, 1e-5, 0, 2048, None, None, None) == 0
+    assert lib.sy_add_rmsnorm_logits(None, None, None, 1e-5, None, 2000, 4, 2048, None, None, None, None) == 1
+    assert lib.sy_add_rmsnorm_logits(None, None, None, 1e-5, None, 64, 0, 2048, None, None, None, None) == 0
+    assert lib.sy_combine_add_rmsnorm(None, None, None, 65, None, None, 1e-5, 4, 2048, None, None, None) == 1
+    assert lib.sy_combine_add_rmsnorm(None, None, None, 8, None, None, 1e-5, 4, 2044, None, None, None) == 1
+    assert lib.sy_combine_add_rmsnorm(None, None, None, 8, None, None, 1e-5, 0, 2048, None, None, None) == 0
     assert lib.sy_qk_norm_rope_cache(None, None, None, 1e-5, 0.0, None, None, 64, None, None, 2, 16, 5, 128, 64, None, None,
                                      None, None) == 1
     assert lib.sy_qk_norm_rope_cache(None, None, None, 1e-5, 0.0, None, None, 64, None, None, 2, 16, 16, 72, 64, None, None,

@@ -42,6 +42,41 @@ def test_add_rmsnorm(N, H):
     assert xo2 is x2 and torch.equal(x2, xo) and torch.equal(h2, h)
 
 
+@pytest.mark.parametrize("N,H,E", [(8, 2048, 64), (64, 2048, 64), (3, 512, 16), (5, 520, 7), (2, 2048, 130)])
+def test_add_rmsnorm_with_router_logits(N, H, E):
+    """The same x_out and h as the plain call, bit for bit, plus the router's logits of h: fp32
+    sums rounded once, compared with the fp32 product of the very same h."""
+    x, d, w = rnd(N, H, seed=1), rnd(N, H, seed=2, std=0.3), 1 + rnd(H, seed=3, std=0.1)
+    router = rnd(E, H, seed=4, std=0.02)
+    ext = kernels.ext()
+    xo, h = ext.add_rmsnorm(x, d, w, 1e-5)
+    xo2, h2, logits = ext.add_rmsnorm(x, d, w, 1e-5, router=router)
+    assert torch.equal(xo2, xo) and torch.equal(h2, h)
+    assert logits.shape == (N, E) and logits.dtype == torch.float16
+    want = h.float() @ router.float().T
+    assert torch.allclose(logits.float(), want, rtol=ULP, atol=1e-4)
+    _, h3, logits3 = ext.add_rmsnorm(x, None, w, 1e-5, router=router)
+    assert torch.allclose(logits3.float(), h3.float() @ router.float().T, rtol=ULP, atol=1e-4)
+
+
+@pytest.mark.parametrize("N,H,E,k", [(8, 2048, 64, 8), (64, 2048, 64, 8), (5, 512, 16, 4), (1, 64, 8, 2), (300, 256, 64, 8)])
+def test_combine_add_rmsnorm(N, H, E, k):
+    """combine, residual add and norm in one launch give the bits of the three launches."""
+    g = torch.Generator().manual_seed(5)
+    idx = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(N)]).int().cuda()
+    wts = torch.rand(N, k, generator=g).half().cuda()
+    ext = kernels.ext()
+    counts, offsets, token, wsorted, pos_of = ext.sort_by_expert(idx, wts, E)
+    y, x, w = rnd(N * k, H, seed=6), rnd(N, H, seed=7), 1 + rnd(H, seed=8, std=0.1)
+    delta = ext.combine(y, pos_of, idx, N)
+    xo, h = ext.add_rmsnorm(x, delta, w, 1e-5)
+    xo2, h2 = ext.combine_add_rmsnorm(y, pos_of, idx, x, w, 1e-5)
+    assert torch.equal(xo2, xo) and torch.equal(h2, h)
+    x3 = x.clone()
+    xo3, h3 = ext.combine_add_rmsnorm(y, pos_of, idx, x3, w, 1e-5, x_out=x3)
+    assert xo3 is x3 and torch.equal(x3, xo) and torch.equal(h3, h)
+
+
 def torch_qk_step(qkv, L, s, cos, sin, positions, clip):
     """q, k (normed, clamped, rotated) and v of one new token, as Decoder.step_static does."""
     B = qkv.shape[0]
