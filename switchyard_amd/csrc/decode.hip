@@ -31,12 +31,14 @@ constexpr int ROW_THREADS = 256;
 constexpr int MAX_CHUNKS = 4;  // 8-half chunks per thread: rows of up to 8192 halves
 
 __device__ __forceinline__ float block_sum(float v, float* lds, int slot_base) {
-  // sum over the 4 wavefronts of a 256-thread workgroup; every thread gets the total
+  // sum over the wavefronts of the workgroup (at most 16); every thread gets the total
   v = wave_sum(v);
-  const int wave = threadIdx.x >> 6;
+  const int wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
   if ((threadIdx.x & 63) == 0) lds[slot_base + wave] = v;
   __syncthreads();
-  return lds[slot_base] + lds[slot_base + 1] + lds[slot_base + 2] + lds[slot_base + 3];
+  float total = 0.f;
+  for (int w = 0; w < nwaves; ++w) total += lds[slot_base + w];
+  return total;
 }
 
 constexpr int ROW_MAX_K = 64;  // choices per token the combining variant ranks in one wavefront
@@ -46,17 +48,19 @@ constexpr int ROW_MAX_K = 64;  // choices per token the combining variant ranks 
 // exactly as the combine kernel leaves it; then x_out = f16(x + delta) and h = the RMS norm
 // of x_out. With LOGITS the normalised row stays in LDS and the four wavefronts also take its
 // dot products with the E rows of the router (fp32 sums, one rounding to f16), so that the
-// router needs no launch of its own.
+// router needs no launch of its own; that variant runs 16 wavefronts, each with the loads of
+// four experts in flight at once, because the router's rows come from L2 one round trip at a
+// time and the trips, not the bytes, are what it waits for.
 template <bool COMBINE, bool LOGITS>
-__global__ void __launch_bounds__(ROW_THREADS)
+__global__ void __launch_bounds__(LOGITS ? 1024 : ROW_THREADS)
 row_kernel(const half_t* x, const half_t* __restrict__ delta, const half_t* __restrict__ y,
            const int* __restrict__ pos_of, const int* __restrict__ idx, int k, const half_t* __restrict__ weight,
            float eps, const half_t* __restrict__ router, int E, int H, half_t* x_out, half_t* __restrict__ h_out,
            half_t* __restrict__ logits) {  // x_out may be x
   extern __shared__ __attribute__((aligned(16))) half_t hs[];  // LOGITS: the normalised row [H]
-  __shared__ float part[4];
+  __shared__ float part[16];
   __shared__ int rows[ROW_MAX_K];
-  const int t = blockIdx.x, tid = threadIdx.x;
+  const int t = blockIdx.x, tid = threadIdx.x, nthreads = blockDim.x;
   const size_t row = (size_t)t * H;
   const int chunks = H >> 3;
   if (COMBINE) {
@@ -77,7 +81,7 @@ row_kernel(const half_t* x, const half_t* __restrict__ delta, const half_t* __re
   float ss = 0.f;
 #pragma unroll
   for (int i = 0; i < MAX_CHUNKS; ++i) {
-    const int c = tid + i * ROW_THREADS;
+    const int c = tid + i * nthreads;
     if (c < chunks) {
       v[i] = *reinterpret_cast<const half8_t*>(x + row + c * 8);
       if (COMBINE) {
@@ -101,7 +105,7 @@ row_kernel(const half_t* x, const half_t* __restrict__ delta, const half_t* __re
   const float rs = rsqrtf(block_sum(ss, part, 0) / (float)H + eps);
 #pragma unroll
   for (int i = 0; i < MAX_CHUNKS; ++i) {
-    const int c = tid + i * ROW_THREADS;
+    const int c = tid + i * nthreads;
     if (c < chunks) {
       const half8_t w = *reinterpret_cast<const half8_t*>(weight + c * 8);
       half8_t h;
@@ -114,27 +118,47 @@ row_kernel(const half_t* x, const half_t* __restrict__ delta, const half_t* __re
   }
   if (!LOGITS) return;
   __syncthreads();
-  // wavefront w takes experts w, w + 4, ...: four at a time, so that 4 loads per lane are in flight
-  const int wave = tid >> 6, lane = tid & 63;
-  for (int e0 = wave; e0 < E; e0 += 16) {
+  // wavefront w takes experts w, w + nwaves, ...: four at a time with every load issued before
+  // the first is used (rows of 2048: 16 loads of 16 bytes per lane)
+  const int wave = tid >> 6, lane = tid & 63, nwaves = nthreads >> 6;
+  for (int e0 = wave; e0 < E; e0 += 4 * nwaves) {
+    const half_t* r[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int e = e0 + nwaves * u;
+      r[u] = router + (size_t)(e < E ? e : e0) * H;
+    }
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int c = lane; c < chunks; c += WAVE) {
-      const half8_t hv = *reinterpret_cast<const half8_t*>(hs + c * 8);
-      half8_t r[4];
+    if (chunks == 4 * WAVE) {
+      half8_t rv[4][4];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int e = e0 + 4 * u;
-        r[u] = *reinterpret_cast<const half8_t*>(router + (size_t)(e < E ? e : e0) * H + c * 8);
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int u = 0; u < 4; ++u) rv[u][i] = *reinterpret_cast<const half8_t*>(r[u] + (lane + WAVE * i) * 8);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const half8_t hv = *reinterpret_cast<const half8_t*>(hs + (lane + WAVE * i) * 8);
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+          for (int j = 0; j < 8; ++j) acc[u] += (float)hv[j] * (float)rv[u][i][j];
       }
+    } else {
+      for (int c = lane; c < chunks; c += WAVE) {
+        const half8_t hv = *reinterpret_cast<const half8_t*>(hs + c * 8);
+        half8_t rv[4];
 #pragma unroll
-      for (int u = 0; u < 4; ++u)
+        for (int u = 0; u < 4; ++u) rv[u] = *reinterpret_cast<const half8_t*>(r[u] + c * 8);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc[u] += (float)hv[j] * (float)r[u][j];
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+          for (int j = 0; j < 8; ++j) acc[u] += (float)hv[j] * (float)rv[u][j];
+      }
     }
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const float total = wave_sum(acc[u]);
-      const int e = e0 + 4 * u;
+      const int e = e0 + nwaves * u;
       if (lane == 0 && e < E) logits[(size_t)t * E + e] = (half_t)total;
     }
   }
@@ -166,7 +190,7 @@ qk_norm_rope_cache_kernel(const half_t* __restrict__ qkv, const half_t* __restri
                           const int64_t* __restrict__ slot_ptr, int heads, int kv_heads, int D, int capacity,
                           half_t* __restrict__ q_out, half_t* __restrict__ kcache, half_t* __restrict__ vcache) {
   extern __shared__ __attribute__((aligned(16))) half_t normed[];  // [qd + kvd] after norm and clamp
-  __shared__ float part[8];
+  __shared__ float part[32];
   const int b = blockIdx.x;
   const int qd = heads * D, kvd = kv_heads * D;
   const half_t* row = qkv + (size_t)b * (qd + 2 * kvd);
@@ -193,7 +217,7 @@ qk_norm_rope_cache_kernel(const half_t* __restrict__ qkv, const half_t* __restri
     }
   }
   const float rq = rsqrtf(block_sum(sq, part, 0) / (float)qd + eps);
-  const float rk = rsqrtf(block_sum(sk, part, 4) / (float)kvd + eps);
+  const float rk = rsqrtf(block_sum(sk, part, 16) / (float)kvd + eps);
 #pragma unroll
   for (int i = 0; i < MAX_CHUNKS; ++i) {
     const int c = threadIdx.x + i * ROW_THREADS;
@@ -398,7 +422,7 @@ extern "C" SY_API int sy_add_rmsnorm_logits(const void* x, const void* delta, co
   SY_REQUIRE(E >= 1 && E <= 1024, "add_rmsnorm_logits: 1 <= E <= 1024 (got %d)", E);
   if (N == 0) return SY_OK;
   SY_REQUIRE(x && weight && h_out && router && logits, "add_rmsnorm_logits: null pointer");
-  row_kernel<false, true><<<N, ROW_THREADS, (size_t)H * sizeof(half_t), (hipStream_t)stream>>>(
+  row_kernel<false, true><<<N, 1024, (size_t)H * sizeof(half_t), (hipStream_t)stream>>>(
       (const half_t*)x, (const half_t*)delta, nullptr, nullptr, nullptr, 0, (const half_t*)weight, eps,
       (const half_t*)router, E, H, (half_t*)x_out, (half_t*)h_out, (half_t*)logits);
   return sy_check_launch("add_rmsnorm_logits");
