@@ -72,6 +72,18 @@ SY_API int sy_decode_attention(const void* q, const void* kcache, const void* vc
                                const int64_t* slot, int B, int heads, int kv_heads, int D, int capacity, void* out,
                                void* stream);
 
+/* sy_qk_norm_rope_cache and sy_decode_attention in one launch (switchyard/model.py:64-84 with
+ * T = 1): every workgroup norms, clamps and rotates its own head of q and of the new key from
+ * `qkv`, attends to the cached keys before `slot` and to the new key and value from registers,
+ * and the first query head of each kv head writes them into the cache at `slot`. Arguments as
+ * for the two entry points; q is not materialised. Results equal theirs up to the order of the
+ * fp32 softmax sums. */
+SY_API int sy_decode_attention_qkv(const void* qkv, const void* q_norm, const void* k_norm, float eps, float clip,
+                                   const void* cos_table, const void* sin_table, int max_positions,
+                                   const int64_t* positions, const int64_t* slot, const uint8_t* real, int B, int heads,
+                                   int kv_heads, int D, int capacity, void* kcache, void* vcache, void* out,
+                                   void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -43,6 +43,9 @@ SIGNATURES = {
     "sy_qk_norm_rope_cache": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_float, _c_void_p, _c_void_p, _c_int,
                                        _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p,
                                        _c_void_p, _c_void_p, _c_void_p]),
+    "sy_decode_attention_qkv": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_float, _c_void_p, _c_void_p, _c_int,
+                                         _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int,
+                                         _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
     "sy_decode_attention": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
                                      _c_int, _c_int, _c_void_p, _c_void_p]),
 }
@@ -281,4 +284,32 @@ class Ext:
         out = torch.empty_like(q)
         self._call(self.lib.sy_decode_attention, q.data_ptr(), kcache.data_ptr(), vcache.data_ptr(), real.data_ptr(),
                    slot.data_ptr(), B, int(heads), kv_heads, D, capacity, out.data_ptr(), _stream())
+        return out
+
+    def decode_attention_qkv(self, qkv, q_norm, k_norm, eps, clip, cos, sin, positions, slot, real, heads, kv_heads,
+                             head_dim, kcache, vcache):
+        """qk_norm_rope_cache and decode_attention in one launch: qkv [B, (heads + 2 kv_heads) D]
+        -> attention output [B, heads D]; the new key and value are written at `slot`."""
+        for t, name in ((qkv, "qkv"), (q_norm, "q_norm"), (k_norm, "k_norm"), (cos, "cos"), (sin, "sin"),
+                        (kcache, "kcache"), (vcache, "vcache")):
+            _check(t, name, torch.float16)
+        _check(positions, "positions", torch.int64)
+        _check(slot, "slot", torch.int64)
+        _check(real, "real", torch.bool)
+        B, D = qkv.shape[0], int(head_dim)
+        if qkv.shape[1] != (heads + 2 * kv_heads) * D or q_norm.numel() != heads * D or k_norm.numel() != kv_heads * D:
+            raise RuntimeError("decode_attention_qkv: qkv / q_norm / k_norm do not match heads, kv_heads and head_dim")
+        if cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] != D:
+            raise RuntimeError("decode_attention_qkv: cos and sin must be [max_positions, head_dim]")
+        if kcache.shape != vcache.shape or kcache.dim() != 4 or tuple(kcache.shape[:2]) != (B, kv_heads) or \
+                kcache.shape[3] != D:
+            raise RuntimeError("decode_attention_qkv: caches must be [B, kv_heads, capacity, head_dim]")
+        capacity = kcache.shape[2]
+        if positions.numel() != B or slot.numel() != 1 or tuple(real.shape) != (B, capacity):
+            raise RuntimeError("decode_attention_qkv: positions [B], slot [1], real [B, capacity]")
+        out = torch.empty((B, heads * D), dtype=torch.float16, device=qkv.device)
+        self._call(self.lib.sy_decode_attention_qkv, qkv.data_ptr(), q_norm.data_ptr(), k_norm.data_ptr(), float(eps),
+                   float(clip or 0.0), cos.data_ptr(), sin.data_ptr(), cos.shape[0], positions.data_ptr(),
+                   slot.data_ptr(), real.data_ptr(), B, int(heads), int(kv_heads), D, capacity, kcache.data_ptr(),
+                   vcache.data_ptr(), out.data_ptr(), _stream())
         return out

@@ -13,7 +13,8 @@
 //   qk_norm_rope_cache    q/k RMS norm over the whole projection, clamp, rotary embedding, and
 //                         the new key and value written into the cache at `slot`
 //   decode_attention      one query per (sequence, head) against the cache: a single pass over
-//                         the keys and values with a running softmax, HBM-bound
+//                         the keys and values with a running softmax, HBM-bound; its _qkv form
+//                         does the work of qk_norm_rope_cache in its own prologue
 //
 // Everything a replayed HIP graph must not bake in (the cache slot, the rotary positions) is
 // read from device memory, so the same launches serve every step.
@@ -285,7 +286,6 @@ __device__ __forceinline__ float key_sum(float v) {
   return v;
 }
 
-constexpr int ATT_UNROLL = 4;        // key groups in flight per wavefront
 constexpr float MASKED = -1.0e30f;   // running maximum before any key was seen
 
 // One workgroup per (sequence, query head), NW wavefronts. A load instruction covers KPL =
@@ -294,57 +294,171 @@ constexpr float MASKED = -1.0e30f;   // running maximum before any key was seen
 // own running softmax (maximum, sum, 8 output dimensions per lane) over the keys it meets, so
 // the key loop has no cross-lane traffic except the score's sum; the KPL x NW partial results
 // are merged once at the end.
+// What the fused variant needs beyond the plain one: the projections' output and what
+// qk_norm_rope_cache takes.
+struct NewToken {
+  const half_t* qkv;      // [B, (heads + 2 kv_heads) D]
+  const half_t* q_norm;   // [heads D]
+  const half_t* k_norm;   // [kv_heads D]
+  const half_t* cos_t;    // [max_positions, D]
+  const half_t* sin_t;
+  const int64_t* positions;
+  half_t* kcache_w;       // the caches again, writable
+  half_t* vcache_w;
+  float eps, clip;
+  int max_positions;
+};
+
+// A head's 16-byte chunk c of a projection, loaded with everything its norm and rotary
+// embedding need, so that the loads are in flight before the norm's scale is known.
 template <int LPK>
-__global__ void decode_attention_kernel(const half_t* __restrict__ q, const half_t* __restrict__ kcache,
-                                        const half_t* __restrict__ vcache, const uint8_t* __restrict__ real,
-                                        const int64_t* __restrict__ slot_ptr, int heads, int kv_heads, int capacity,
-                                        float scale_log2e, half_t* __restrict__ out) {
+struct HeadChunk {
+  half8_t mine, other, wm, wo;
+  __device__ __forceinline__ void load(const half_t* head, const half_t* norm_w, int c) {
+    const int partner = c ^ (LPK / 2);
+    mine = *reinterpret_cast<const half8_t*>(head + c * 8);
+    other = *reinterpret_cast<const half8_t*>(head + partner * 8);
+    wm = *reinterpret_cast<const half8_t*>(norm_w + c * 8);
+    wo = *reinterpret_cast<const half8_t*>(norm_w + partner * 8);
+  }
+  // RMS norm (scale rs), clamp and rotary embedding, with the roundings of qk_norm_rope_cache
+  __device__ __forceinline__ half8_t finish(float rs, float clip, half8_t cc, half8_t ss, int c) const {
+    const bool low = c < LPK / 2;
+    half8_t o;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const half_t a = clamp_f16((half_t)((float)wm[j] * (float)(half_t)((float)mine[j] * rs)), clip);
+      const half_t r = clamp_f16((half_t)((float)wo[j] * (float)(half_t)((float)other[j] * rs)), clip);
+      o[j] = rotary_f16(a, low ? -r : r, cc[j], ss[j]);
+    }
+    return o;
+  }
+};
+
+// A batch of UNROLL key groups of one wavefront: 16 bytes of key and of value per lane each.
+template <int UNROLL>
+struct KeyBatch {
+  half8_t kk[UNROLL], vv[UNROLL];
+  bool ok[UNROLL];
+};
+
+// FUSED: the query is taken from the projections' output (norm over the whole q and k rows of
+// the sequence, clamp, rotary embedding: the work of qk_norm_rope_cache, redone by every
+// workgroup for its own head, which costs two 4 KB reads from L2), the new key and value are
+// used from registers as the last key, and the first query head of each kv head writes them
+// into the cache; the loop then covers the cached keys before `slot` only.
+// The first batch of keys and values is requested before any of that. (Requesting each further
+// batch while the previous one is multiplied costs registers, hence resident wavefronts, and
+// with them bandwidth: 67.5 us against 55.3 us at 64 sequences x 16 heads x 536 keys.)
+// NW wavefronts per workgroup, each with a batch of UNROLL key groups in flight: 16 wavefronts
+// when there are few (sequence, head) pairs, so that the cache is still read by many, 4 when
+// the pairs fill the chip.
+template <int LPK, bool FUSED, int NW, int UNROLL>
+__global__ void __launch_bounds__(NW * WAVE)
+decode_attention_kernel(const half_t* __restrict__ q, const half_t* kcache, const half_t* vcache,
+                                        const uint8_t* __restrict__ real, const int64_t* __restrict__ slot_ptr,
+                                        int heads, int kv_heads, int capacity, float scale_log2e,
+                                        half_t* __restrict__ out, NewToken nt) {
   constexpr int D = LPK * 8, KPL = WAVE / LPK;
   extern __shared__ float merge[];  // [NW][D + 2]: accumulators, maximum, sum
-  const int NW = blockDim.x >> 6;
+  __shared__ float part[32];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int sub = lane / LPK, c = lane % LPK;
   const int b = blockIdx.x / heads, qh = blockIdx.x % heads;
-  const int kvh = qh / (heads / kv_heads);
-  long n = (long)*slot_ptr + 1;
+  const int group = heads / kv_heads, kvh = qh / group;
+  const long slot = (long)*slot_ptr;
+  long n = FUSED ? slot : slot + 1;   // cached keys the loop visits
   n = n < 0 ? 0 : n > capacity ? capacity : n;
-
-  const half8_t qv = *reinterpret_cast<const half8_t*>(q + ((size_t)b * heads + qh) * D + c * 8);
-  float qf[8];
-#pragma unroll
-  for (int j = 0; j < 8; ++j) qf[j] = (float)qv[j] * scale_log2e;
   const size_t base = ((size_t)b * kv_heads + kvh) * (size_t)capacity * D + c * 8;
   const uint8_t* rl = real + (size_t)b * capacity;
+  const half8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  const int groups = ((int)n + KPL - 1) / KPL, stride = NW * UNROLL;
+
+  auto fetch = [&](KeyBatch<UNROLL>& kb, int g0) {
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int key = (g0 + u * NW) * KPL + sub;
+      kb.ok[u] = key < n;
+      kb.kk[u] = zero8;
+      kb.vv[u] = zero8;
+      if (kb.ok[u]) {
+        kb.kk[u] = *reinterpret_cast<const half8_t*>(kcache + base + (size_t)key * D);
+        kb.vv[u] = *reinterpret_cast<const half8_t*>(vcache + base + (size_t)key * D);
+        kb.ok[u] = rl[key] != 0;
+      }
+    }
+  };
+  KeyBatch<UNROLL> ka;
+  fetch(ka, wave);   // requested before the prologue, so that the two waits overlap
+
+  float qf[8];
+  half8_t knew = zero8, vnew = zero8;
+  if (FUSED) {
+    const int qd = heads * D, kvd = kv_heads * D;
+    const half_t* row = nt.qkv + (size_t)b * (qd + 2 * kvd);
+    long pos = (long)nt.positions[b];
+    pos = pos < 0 ? 0 : pos >= nt.max_positions ? nt.max_positions - 1 : pos;
+    HeadChunk<LPK> hq, hk;
+    hq.load(row + qh * D, nt.q_norm + qh * D, c);
+    hk.load(row + qd + kvh * D, nt.k_norm + kvh * D, c);
+    vnew = *reinterpret_cast<const half8_t*>(row + qd + kvd + kvh * D + c * 8);
+    const half8_t cc = *reinterpret_cast<const half8_t*>(nt.cos_t + (size_t)pos * D + c * 8);
+    const half8_t ss = *reinterpret_cast<const half8_t*>(nt.sin_t + (size_t)pos * D + c * 8);
+    float sq = 0.f, sk = 0.f;
+    for (int i = threadIdx.x; i < (qd >> 3); i += blockDim.x) {
+      const half8_t v = *reinterpret_cast<const half8_t*>(row + i * 8);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) sq += (float)v[j] * (float)v[j];
+    }
+    for (int i = threadIdx.x; i < (kvd >> 3); i += blockDim.x) {
+      const half8_t v = *reinterpret_cast<const half8_t*>(row + qd + i * 8);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) sk += (float)v[j] * (float)v[j];
+    }
+    // both sums through one barrier
+    sq = wave_sum(sq);
+    sk = wave_sum(sk);
+    if (lane == 0) {
+      part[wave] = sq;
+      part[16 + wave] = sk;
+    }
+    __syncthreads();
+    sq = sk = 0.f;
+    for (int w = 0; w < NW; ++w) {
+      sq += part[w];
+      sk += part[16 + w];
+    }
+    const float rq = rsqrtf(sq / (float)qd + nt.eps), rk = rsqrtf(sk / (float)kvd + nt.eps);
+    const half8_t qv = hq.finish(rq, nt.clip, cc, ss, c);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) qf[j] = (float)qv[j] * scale_log2e;
+    knew = hk.finish(rk, nt.clip, cc, ss, c);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) vnew[j] = clamp_f16(vnew[j], nt.clip);
+    if (slot >= 0 && slot < capacity && qh % group == 0 && wave == 0 && sub == 0) {
+      const size_t at = (((size_t)b * kv_heads + kvh) * capacity + slot) * D + c * 8;
+      *reinterpret_cast<half8_t*>(nt.kcache_w + at) = knew;
+      *reinterpret_cast<half8_t*>(nt.vcache_w + at) = vnew;
+    }
+  } else {
+    const half8_t qv = *reinterpret_cast<const half8_t*>(q + ((size_t)b * heads + qh) * D + c * 8);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) qf[j] = (float)qv[j] * scale_log2e;
+  }
 
   float m = MASKED, l = 0.f, acc[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) acc[j] = 0.f;
-  const half8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
 
-  const int groups = ((int)n + KPL - 1) / KPL;
-  for (int g0 = wave; g0 < groups; g0 += NW * ATT_UNROLL) {
-    half8_t kk[ATT_UNROLL], vv[ATT_UNROLL];
-    bool ok[ATT_UNROLL];
+  auto consume = [&](const KeyBatch<UNROLL>& kb) {
+    float s[UNROLL], mx = m;
 #pragma unroll
-    for (int u = 0; u < ATT_UNROLL; ++u) {
-      const int key = (g0 + u * NW) * KPL + sub;
-      ok[u] = key < n;
-      kk[u] = zero8;
-      vv[u] = zero8;
-      if (ok[u]) {
-        kk[u] = *reinterpret_cast<const half8_t*>(kcache + base + (size_t)key * D);
-        vv[u] = *reinterpret_cast<const half8_t*>(vcache + base + (size_t)key * D);
-        ok[u] = rl[key] != 0;
-      }
-    }
-    float s[ATT_UNROLL], mx = m;
-#pragma unroll
-    for (int u = 0; u < ATT_UNROLL; ++u) {
+    for (int u = 0; u < UNROLL; ++u) {
       float d = 0.f;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) d += qf[j] * (float)kk[u][j];
+      for (int j = 0; j < 8; ++j) d += qf[j] * (float)kb.kk[u][j];
       s[u] = key_sum<LPK>(d);
-      if (ok[u]) mx = fmaxf(mx, s[u]);
+      if (kb.ok[u]) mx = fmaxf(mx, s[u]);
     }
     const float alpha = __builtin_amdgcn_exp2f(m - mx);
     m = mx;
@@ -352,12 +466,32 @@ __global__ void decode_attention_kernel(const half_t* __restrict__ q, const half
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[j] *= alpha;
 #pragma unroll
-    for (int u = 0; u < ATT_UNROLL; ++u) {
-      const float p = ok[u] ? __builtin_amdgcn_exp2f(s[u] - mx) : 0.f;
+    for (int u = 0; u < UNROLL; ++u) {
+      const float p = kb.ok[u] ? __builtin_amdgcn_exp2f(s[u] - mx) : 0.f;
       l += p;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) acc[j] += p * (float)vv[u][j];
+      for (int j = 0; j < 8; ++j) acc[j] += p * (float)kb.vv[u][j];
     }
+  };
+  for (int g0 = wave; g0 < groups; g0 += stride) {
+    if (g0 != wave) fetch(ka, g0);
+    consume(ka);
+  }
+
+  if (FUSED && wave == 0 && slot >= 0 && slot < capacity) {
+    // the new token's own key and value, from registers: one more key for the first key group
+    float d = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) d += qf[j] * (float)knew[j];
+    const float sc = key_sum<LPK>(d);
+    const bool ok = sub == 0 && rl[slot] != 0;
+    const float mx = ok ? fmaxf(m, sc) : m;
+    const float alpha = __builtin_amdgcn_exp2f(m - mx);
+    const float p = ok ? __builtin_amdgcn_exp2f(sc - mx) : 0.f;
+    m = mx;
+    l = l * alpha + p;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = acc[j] * alpha + p * (float)vnew[j];
   }
 
   // ---- merge the KPL key groups of the wavefront (lanes with equal c)
@@ -478,9 +612,37 @@ extern "C" SY_API int sy_decode_attention(const void* q, const void* kcache, con
   const int waves = pairs >= 2l * sy_compute_units() ? 4 : 16;
   const size_t lds = (size_t)waves * (D + 2) * sizeof(float);
   const float scale_log2e = 1.4426950408889634f / sqrtf((float)D);
-  auto kern = D == 128 ? decode_attention_kernel<16> : decode_attention_kernel<8>;
+  auto kern = D == 128 ? (waves == 4 ? decode_attention_kernel<16, false, 4, 4> : decode_attention_kernel<16, false, 16, 4>)
+                       : (waves == 4 ? decode_attention_kernel<8, false, 4, 4> : decode_attention_kernel<8, false, 16, 4>);
   kern<<<(unsigned)pairs, waves * WAVE, lds, (hipStream_t)stream>>>((const half_t*)q, (const half_t*)kcache,
                                                                    (const half_t*)vcache, real, slot, heads, kv_heads,
-                                                                   capacity, scale_log2e, (half_t*)out);
+                                                                   capacity, scale_log2e, (half_t*)out, NewToken{});
   return sy_check_launch("decode_attention");
+}
+
+extern "C" SY_API int sy_decode_attention_qkv(const void* qkv, const void* q_norm, const void* k_norm, float eps, float clip,
+                                              const void* cos_table, const void* sin_table, int max_positions,
+                                              const int64_t* positions, const int64_t* slot, const uint8_t* real, int B,
+                                              int heads, int kv_heads, int D, int capacity, void* kcache, void* vcache,
+                                              void* out, void* stream) {
+  SY_REQUIRE(B >= 0 && heads >= 1 && kv_heads >= 1 && heads % kv_heads == 0,
+             "decode_attention_qkv: B = %d, heads = %d, kv_heads = %d", B, heads, kv_heads);
+  SY_REQUIRE(D == 64 || D == 128, "decode_attention_qkv: head_dim must be 64 or 128 (got %d)", D);
+  SY_REQUIRE(capacity >= 1 && max_positions >= 1, "decode_attention_qkv: capacity = %d, max_positions = %d", capacity,
+             max_positions);
+  if (B == 0) return SY_OK;
+  SY_REQUIRE(qkv && q_norm && k_norm && cos_table && sin_table && positions && slot && real && kcache && vcache && out,
+             "decode_attention_qkv: null pointer");
+  const long pairs = (long)B * heads;
+  const int waves = pairs >= 2l * sy_compute_units() ? 4 : 16;
+  const size_t lds = (size_t)waves * (D + 2) * sizeof(float);
+  const float scale_log2e = 1.4426950408889634f / sqrtf((float)D);
+  NewToken nt{(const half_t*)qkv, (const half_t*)q_norm, (const half_t*)k_norm, (const half_t*)cos_table,
+              (const half_t*)sin_table, positions, (half_t*)kcache, (half_t*)vcache, eps, clip, max_positions};
+  auto kern = D == 128 ? (waves == 4 ? decode_attention_kernel<16, true, 4, 4> : decode_attention_kernel<16, true, 16, 4>)
+                       : (waves == 4 ? decode_attention_kernel<8, true, 4, 4> : decode_attention_kernel<8, true, 16, 4>);
+  kern<<<(unsigned)pairs, waves * WAVE, lds, (hipStream_t)stream>>>(nullptr, (const half_t*)kcache, (const half_t*)vcache,
+                                                                   real, slot, heads, kv_heads, capacity, scale_log2e,
+                                                                   (half_t*)out, nt);
+  return sy_check_launch("decode_attention_qkv");
 }

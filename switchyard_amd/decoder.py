@@ -261,8 +261,9 @@ class Decoder:
     @torch.no_grad()
     def step_fused(self, tok, cache, slot, keys=None):
         """The same step as `step_static` on the decode kernels: residual add + RMS norm, the
-        stacked q/k/v projection, norm + rotary + cache write, attention over the cache, the
-        output projection, and the MoE hook; every projection streams its weights once."""
+        stacked q/k/v projection, attention over the cache (with the q/k norm, the rotary
+        embedding and the cache write in its prologue), the output projection, and the MoE
+        hook; every projection streams its weights once."""
         from . import kernels
 
         s, W, E = self.s, self.w, kernels.ext()
@@ -274,10 +275,9 @@ class Decoder:
         for i in range(s.layers):
             L = W["layers"][i]
             after = W["layers"][i + 1]["attn_norm"] if i + 1 < s.layers else W["final_norm"]
-            q = E.qk_norm_rope_cache(kernels.dense(xn, wqkv[i]), L["q_norm"], L["k_norm"], s.rms_eps, s.clip_qkv,
-                                     self.cos, self.sin, positions, slot, s.heads, s.kv_heads, s.head_dim,
-                                     cache.k[i], cache.v[i])
-            a = E.decode_attention(q, cache.k[i], cache.v[i], cache.real, slot, s.heads)
+            a = E.decode_attention_qkv(kernels.dense(xn, wqkv[i]), L["q_norm"], L["k_norm"], s.rms_eps, s.clip_qkv,
+                                       self.cos, self.sin, positions, slot, cache.real, s.heads, s.kv_heads,
+                                       s.head_dim, cache.k[i], cache.v[i])
             o = kernels.dense(a, L["wo"])
             if self._own_moe and s.experts <= 1024 and s.top_k <= 64:
                 # the router's logits come out of the norm's launch, and combine goes into the next norm's

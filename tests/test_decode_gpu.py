@@ -152,6 +152,43 @@ def test_decode_attention(B, heads, kv_heads, hd, cap, slot_at):
     assert torch.allclose(out.float(), want.reshape(B, heads * hd), rtol=2 * ULP, atol=1e-3)
 
 
+@pytest.mark.parametrize("B,heads,kv_heads,hd,cap,slot_at,clip", [
+    (8, 16, 16, 128, 640, 600, None), (64, 16, 16, 128, 200, 199, 0.5), (3, 8, 2, 64, 77, 50, None),
+    (2, 4, 4, 128, 9, 0, None), (2, 4, 1, 64, 33, 2, 1.0), (40, 16, 4, 64, 130, 129, None)])
+def test_attention_with_the_norm_and_rotary_in_its_prologue(B, heads, kv_heads, hd, cap, slot_at, clip):
+    """One launch against the two it replaces: the same cache contents bit for bit, the same
+    output up to the order of the fp32 softmax sums (one fp16 rounding)."""
+    s = D.Shape(hidden=512, heads=heads, kv_heads=kv_heads, head_dim=hd, clip_qkv=clip)
+    max_pos = 700
+    dec = D.Decoder(s, {"embed": torch.zeros(1, 8, dtype=torch.float16, device="cuda"), "layers": []}, moe=lambda i, h: h,
+                    max_positions=max_pos, attention="torch")
+    qd, kvd = heads * hd, kv_heads * hd
+    g = torch.Generator().manual_seed(21)
+    qkv = rnd(B, qd + 2 * kvd, seed=22, std=0.7)
+    qn, kn = 1 + rnd(qd, seed=23, std=0.1), 1 + rnd(kvd, seed=24, std=0.1)
+    positions = torch.randint(0, max_pos, (B,), generator=g).cuda()
+    slot = torch.tensor([slot_at], device="cuda")
+    real = torch.rand(B, cap, generator=g) > 0.2
+    real[:, slot_at] = True
+    real = real.cuda()
+    kc, vc = rnd(B, kv_heads, cap, hd, seed=25), rnd(B, kv_heads, cap, hd, seed=26)
+    kc2, vc2 = kc.clone(), vc.clone()
+    ext = kernels.ext()
+    q = ext.qk_norm_rope_cache(qkv, qn, kn, s.rms_eps, clip, dec.cos, dec.sin, positions, slot, heads, kv_heads, hd, kc, vc)
+    want = ext.decode_attention(q, kc, vc, real, slot, heads)
+    got = ext.decode_attention_qkv(qkv, qn, kn, s.rms_eps, clip, dec.cos, dec.sin, positions, slot, real, heads, kv_heads,
+                                   hd, kc2, vc2)
+    assert torch.equal(kc2, kc) and torch.equal(vc2, vc)
+    assert torch.allclose(got.float(), want.float(), rtol=2 * ULP, atol=1e-3)
+    # a slot past the cache: nothing is written, every cached key is visible
+    slot_out = torch.tensor([cap], device="cuda")
+    got = ext.decode_attention_qkv(qkv, qn, kn, s.rms_eps, clip, dec.cos, dec.sin, positions, slot_out, real, heads,
+                                   kv_heads, hd, kc2, vc2)
+    assert torch.equal(kc2, kc) and torch.equal(vc2, vc)
+    want = ext.decode_attention(q, kc, vc, real, slot_out, heads)
+    assert torch.allclose(got.float(), want.float(), rtol=2 * ULP, atol=1e-3)
+
+
 def test_decode_attention_without_a_real_key_gives_zeros():
     B, heads, hd, cap = 2, 4, 64, 16
     q, kc, vc = rnd(B, heads * hd), rnd(B, heads, cap, hd), rnd(B, heads, cap, hd)
