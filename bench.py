@@ -296,6 +296,11 @@ def run_decode(args):
         tm = {}
         graph_tokens, first = model.generate_graph(prompts, args.new_tokens + 1, return_first_logits=True, timings=tm)
         t_prefill, t_decode, steps = tm["prefill_s"], tm["decode_s"], tm["decode_steps"]
+        if args.graph_only:   # profiling runs: nothing but the prefill and the replayed steps
+            print(json.dumps({"bench": "decode", "batch": B, "prompt_len": args.prompt_len, "new_tokens": steps,
+                              "decode_tok_per_s": B * steps / t_decode, "ms_per_step": t_decode * 1e3 / steps,
+                              "prefill_ms": t_prefill * 1e3, "model": name}), flush=True)
+            continue
         # the eager loop (one Python-driven step per token) for comparison, fewer tokens
         cache = D.KVCache(s, B, args.prompt_len + 16, torch.float16, dev)
         logits = model.forward(tokens, cache)[:, -1]
@@ -349,6 +354,8 @@ def main():
                     help="decode: an OLMoE checkpoint directory (config.json + safetensors) instead of random weights")
     ap.add_argument("--prompt-len", type=int, default=512)
     ap.add_argument("--new-tokens", type=int, default=128)
+    ap.add_argument("--graph-only", action="store_true",
+                    help="decode: only the prefill and the graph-replayed steps (profiling runs)")
     ap.add_argument("--decode-loop-steps", type=int, default=8,
                     help="decode steps to time with the per-expert loop in the hook (0: skip)")
     args = ap.parse_args()
