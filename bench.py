@@ -12,7 +12,10 @@ a decoder does, so that no step finds its weights in the 256 MB last-level cache
 
 Prints ONE JSON line with the metric, a `roofline` object for the dominant kernel (the
 gate/up projection: two thirds of the weight bytes), timed per launch with events on the
-launch stream, and a `cpu_baseline` object: the per-expert PyTorch loop on this host's cores."""
+launch stream, a `cpu_baseline` object: the per-expert PyTorch loop on this host's cores, and (in
+the default configuration) a `decode` object: tokens/s of the full 16-layer model's greedy decode
+at batch 8 and 64, the second half of the reference's headline (`--decode 8,64` gives the detailed
+lines with the comparison against the per-expert loop in the hook)."""
 
 import argparse
 import json
@@ -101,6 +104,28 @@ def cpu_loop_baseline(h, router, gu, dn, used, reps=5):
             "us_per_layer": t * 1e6}
 
 
+def decode_rates(batches=(8, 64), prompt_len=512, new_tokens=128):
+    """The other half of the headline metric: greedy decode of the full OLMoE-1B-7B-shaped model
+    (16 layers, random fp16 weights), HIP-graph replay of the step, tokens/s per batch size."""
+    from switchyard_amd import decoder as D
+
+    s = D.OLMOE_1B_7B
+    w = D.random_weights(s, device="cuda:0", seed=0)
+    model = D.Decoder(s, w, max_positions=prompt_len + new_tokens + 8)
+    out = {"model": "OLMoE-1B-7B shape, 16 layers, random-init fp16", "prompt_len": prompt_len,
+           "new_tokens": new_tokens, "step": "HIP-graph replay of Decoder.step_fused"}
+    for B in batches:
+        prompts = torch.randint(3, s.vocab, (B, prompt_len), generator=torch.Generator().manual_seed(0)).tolist()
+        model.generate(prompts, 4)
+        torch.cuda.synchronize()
+        tm = {}
+        model.generate_graph(prompts, new_tokens + 1, timings=tm)
+        out[f"b{B}"] = {"tok_per_s": B * tm["decode_steps"] / tm["decode_s"],
+                        "ms_per_step": tm["decode_s"] * 1e3 / tm["decode_steps"],
+                        "prefill_tok_per_s": B * prompt_len / tm["prefill_s"]}
+    return out
+
+
 def run_default(args):
     from switchyard_amd import kernels
 
@@ -187,6 +212,15 @@ def run_default(args):
     roof["algorithmic_per_launch"] = alg
 
     cpu = None if args.no_cpu else cpu_loop_baseline(h_cpu, *cpu_layers[0], used[0])
+    n_layers = len(layers)
+    decode = None
+    if not args.no_cpu and N == 8 and mode == "auto":   # the default run reports the whole metric
+        del layers, rot, router, gu, dn
+        torch.cuda.empty_cache()
+        try:
+            decode = decode_rates()
+        except Exception as exc:  # the layer figures above stand on their own
+            decode = {"error": f"{type(exc).__name__}: {exc}"}
 
     line = {
         "metric": "OLMoE MoE-layer expert-weight GB/s", "value": value, "unit": "GB/s", "n_gpus": 1,
@@ -195,13 +229,13 @@ def run_default(args):
         "data": "synthetic",
         "config": {"workload": f"olmoe_moe_layer_{'decode' if N <= 64 else 'prefill'}_{N}tok", "tokens": N,
                    "experts": E, "top_k": TOPK, "hidden": H, "expert_width": I, "mode": mode,
-                   "layers_rotated": len(layers), "experts_used_mean": used_mean, "spin_up_ms": SPIN_UP_MS},
+                   "layers_rotated": n_layers, "experts_used_mean": used_mean, "spin_up_ms": SPIN_UP_MS},
         "us_per_layer": ms_per_step * 1e3, "us_per_layer_event_median": ev_med * 1e3,
         "frac_of_hbm_peak": value / HBM_PEAK_GBS,
         "tflops": N * TOPK * 6 * H * I / (ms_per_step / 1e3) / 1e12,
         "vs_baseline_note": "published figure is the reference's on one Tesla T4 (320 GB/s)",
         "gpu": torch.cuda.get_device_name(0),
-        "roofline": roof, "cpu_baseline": cpu,
+        "roofline": roof, "cpu_baseline": cpu, "decode": decode,
     }
     print(json.dumps(line), flush=True)
 
@@ -348,7 +382,8 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run a plain 512 MiB device copy 5 times (a kernel of known traffic, to scale "
                          "rocprofv3's FETCH_SIZE / WRITE_SIZE readings)")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg (profiling runs)")
+    ap.add_argument("--no-cpu", action="store_true",
+                    help="skip the CPU baseline and the full-model decode legs (profiling runs)")
     ap.add_argument("--decode", default=None, help='full-model greedy decode at these batch sizes, e.g. "8,64"')
     ap.add_argument("--checkpoint", default=None,
                     help="decode: an OLMoE checkpoint directory (config.json + safetensors) instead of random weights")
