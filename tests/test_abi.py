@@ -123,3 +123,19 @@ def test_host_wrappers_refuse_cpu_tensors():
         kernels.ext().route(torch.zeros(4, 64, dtype=torch.float16), 8, False)
     with pytest.raises(ValueError, match="unknown mode"):
         kernels.ffn(torch.zeros(1, 8), None, None, None, None, None, torch.zeros(1, 8, 8), 1, "nope")
+
+
+def test_bench_refuses_more_than_one_gpu_and_needs_a_gpu():
+    """The benchmark is a one-GPU measurement: --gpus 2 ends with a message, before any device
+    is touched; without a GPU the default run says so instead of falling back to the CPU."""
+    import subprocess
+    import sys
+
+    bench = os.path.join(ROOT, "bench.py")
+    two = subprocess.run([sys.executable, bench, "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert two.returncode != 0 and "one GPU" in two.stderr
+    import torch
+
+    if not torch.cuda.is_available():
+        one = subprocess.run([sys.executable, bench], capture_output=True, text=True, timeout=120)
+        assert one.returncode != 0 and "no GPU" in one.stderr
