@@ -27,6 +27,14 @@ extern "C" {
 SY_API int sy_add_rmsnorm(const void* x, const void* delta, const void* weight, float eps, int N, int H, void* x_out,
                           void* h_out, void* stream);
 
+/* The embedding lookup and the first RMS norm of a step in one launch; replaces F.embedding
+ * (switchyard/model.py:111) followed by rmsnorm() (:119).
+ * tokens int64 [N] (values outside [0, vocab) are clamped); embed f16 [vocab, H]; weight f16 [H]
+ * -> x_out f16 [N,H] = embed[tokens], h_out f16 [N,H] = its RMS norm as sy_add_rmsnorm.
+ * Limits: as sy_add_rmsnorm. */
+SY_API int sy_embed_rmsnorm(const int64_t* tokens, const void* embed, int vocab, const void* weight, float eps, int N,
+                            int H, void* x_out, void* h_out, void* stream);
+
 /* sy_add_rmsnorm that also takes the router's logits of the normalised rows, so that the router
  * GEMM of the MoE layer (`F.linear(h, router)`, switchyard/kernels.py:30-32 after
  * switchyard/model.py:121) needs no launch of its own at decode.
@@ -76,13 +84,26 @@ SY_API int sy_decode_attention(const void* q, const void* kcache, const void* vc
  * T = 1): every workgroup norms, clamps and rotates its own head of q and of the new key from
  * `qkv`, attends to the cached keys before `slot` and to the new key and value from registers,
  * and the first query head of each kv head writes them into the cache at `slot`. Arguments as
- * for the two entry points; q is not materialised. Results equal theirs up to the order of the
- * fp32 softmax sums. */
+ * for the two entry points; q is not materialised. The new token is a real one by definition:
+ * `real` is read for the positions before `slot` and real[:, slot] is SET to 1 (the
+ * `cache.valid[:, start:start+T] = valid` of switchyard/model.py:98 for T = 1), so `real` is
+ * in/out here. Results equal the two entry points' (with real[:, slot] = 1) up to the order of
+ * the fp32 softmax sums. */
 SY_API int sy_decode_attention_qkv(const void* qkv, const void* q_norm, const void* k_norm, float eps, float clip,
                                    const void* cos_table, const void* sin_table, int max_positions,
-                                   const int64_t* positions, const int64_t* slot, const uint8_t* real, int B, int heads,
+                                   const int64_t* positions, const int64_t* slot, uint8_t* real, int B, int heads,
                                    int kv_heads, int D, int capacity, void* kcache, void* vcache, void* out,
                                    void* stream);
+
+/* The end of a greedy decode step in one launch; replaces `logits.argmax(-1)`, the append to
+ * the output and the cache counters' increments of generate() / finish()
+ * (switchyard/model.py:154-157,123-124) for T = 1.
+ * logits f16 [B,V] -> tok int64 [B] = arg-max of each row (the lowest index among equal
+ * maxima); out int64 [B, out_stride]: out[b, next_position[b] - base_position[b]] = tok[b] when
+ * that column exists; next_position int64 [B] += 1; slot int64 [1] += 1.
+ * base_position int64 [B] is what next_position held when column 0 was due. */
+SY_API int sy_greedy_advance(const void* logits, int B, int V, int64_t* tok, int64_t* out, int out_stride,
+                             const int64_t* base_position, int64_t* next_position, int64_t* slot, void* stream);
 
 #ifdef __cplusplus
 }

@@ -36,6 +36,10 @@ SIGNATURES = {
     "sy_combine": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p]),
     "sy_add_rmsnorm": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_int, _c_int, _c_void_p, _c_void_p,
                                 _c_void_p]),
+    "sy_embed_rmsnorm": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_float, _c_int, _c_int, _c_void_p, _c_void_p,
+                                  _c_void_p]),
+    "sy_greedy_advance": (_c_int, [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
+                                   _c_void_p, _c_void_p]),
     "sy_add_rmsnorm_logits": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_int, _c_int,
                                        _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
     "sy_combine_add_rmsnorm": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_float, _c_int,
@@ -223,6 +227,34 @@ class Ext:
                    router.shape[0], N, H, o_ptr, h.data_ptr(), logits.data_ptr(), _stream())
         return first, h, logits
 
+    def embed_rmsnorm(self, tokens, embed, weight, eps):
+        """tokens int64 [N] -> (embed[tokens], weight * rmsnorm(embed[tokens])) in one launch."""
+        _check(tokens, "tokens", torch.int64)
+        _check(embed, "embed", torch.float16)
+        _check(weight, "weight", torch.float16)
+        N, (vocab, H) = tokens.numel(), embed.shape
+        if weight.numel() != H:
+            raise RuntimeError("embed_rmsnorm: weight must have H entries")
+        x = torch.empty((N, H), dtype=torch.float16, device=embed.device)
+        h = torch.empty_like(x)
+        self._call(self.lib.sy_embed_rmsnorm, tokens.data_ptr(), embed.data_ptr(), vocab, weight.data_ptr(), float(eps), N,
+                   H, x.data_ptr(), h.data_ptr(), _stream())
+        return x, h
+
+    def greedy_advance(self, logits, tok, out, base_position, next_position, slot):
+        """The end of a greedy step, in place: tok[b] = argmax(logits[b]) (lowest index among equal
+        maxima), out[b, next_position[b] - base_position[b]] = tok[b], next_position += 1, slot += 1."""
+        _check(logits, "logits", torch.float16)
+        for t, name in ((tok, "tok"), (out, "out"), (base_position, "base_position"), (next_position, "next_position"),
+                        (slot, "slot")):
+            _check(t, name, torch.int64)
+        B, V = logits.shape
+        if tok.numel() != B or out.dim() != 2 or out.shape[0] != B or base_position.numel() != B or \
+                next_position.numel() != B or slot.numel() != 1:
+            raise RuntimeError("greedy_advance: tok / out / positions must have one entry (row) per row of logits")
+        self._call(self.lib.sy_greedy_advance, logits.data_ptr(), B, V, tok.data_ptr(), out.data_ptr(), out.shape[1],
+                   base_position.data_ptr(), next_position.data_ptr(), slot.data_ptr(), _stream())
+
     def combine_add_rmsnorm(self, y, pos_of, idx, x, weight, eps, x_out=None):
         """combine(y, pos_of, idx) added to x [N, H] and normalised in one launch ->
         (x + combine, weight * rmsnorm(x + combine)); x_out may be x."""
@@ -289,7 +321,8 @@ class Ext:
     def decode_attention_qkv(self, qkv, q_norm, k_norm, eps, clip, cos, sin, positions, slot, real, heads, kv_heads,
                              head_dim, kcache, vcache):
         """qk_norm_rope_cache and decode_attention in one launch: qkv [B, (heads + 2 kv_heads) D]
-        -> attention output [B, heads D]; the new key and value are written at `slot`."""
+        -> attention output [B, heads D]; the new key and value are written at `slot`, and
+        real[:, slot] is set (the new token is a real one)."""
         for t, name in ((qkv, "qkv"), (q_norm, "q_norm"), (k_norm, "k_norm"), (cos, "cos"), (sin, "sin"),
                         (kcache, "kcache"), (vcache, "vcache")):
             _check(t, name, torch.float16)

@@ -57,13 +57,20 @@ __global__ void __launch_bounds__(LOGITS ? 1024 : ROW_THREADS)
 row_kernel(const half_t* x, const half_t* __restrict__ delta, const half_t* __restrict__ y,
            const int* __restrict__ pos_of, const int* __restrict__ idx, int k, const half_t* __restrict__ weight,
            float eps, const half_t* __restrict__ router, int E, int H, half_t* x_out, half_t* __restrict__ h_out,
-           half_t* __restrict__ logits) {  // x_out may be x
+           half_t* __restrict__ logits, const int64_t* __restrict__ gather, int src_rows) {  // x_out may be x
   extern __shared__ __attribute__((aligned(16))) half_t hs[];  // LOGITS: the normalised row [H]
   __shared__ float part[16];
   __shared__ int rows[ROW_MAX_K];
   const int t = blockIdx.x, tid = threadIdx.x, nthreads = blockDim.x;
   const size_t row = (size_t)t * H;
   const int chunks = H >> 3;
+  // the input row: row t of x, or (an embedding lookup) the row of x that gather[t] names
+  const half_t* xrow = x + row;
+  if (gather) {
+    long g = (long)gather[t];
+    g = g < 0 ? 0 : g >= src_rows ? src_rows - 1 : g;
+    xrow = x + (size_t)g * H;
+  }
   if (COMBINE) {
     // rank the k choices by (expert id, slot); rows[] lists their rows of y in that order
     if (tid < WAVE) {
@@ -84,7 +91,7 @@ row_kernel(const half_t* x, const half_t* __restrict__ delta, const half_t* __re
   for (int i = 0; i < MAX_CHUNKS; ++i) {
     const int c = tid + i * nthreads;
     if (c < chunks) {
-      v[i] = *reinterpret_cast<const half8_t*>(x + row + c * 8);
+      v[i] = *reinterpret_cast<const half8_t*>(xrow + c * 8);
       if (COMBINE) {
         float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         for (int j = 0; j < k; ++j) {
@@ -305,6 +312,7 @@ struct NewToken {
   const int64_t* positions;
   half_t* kcache_w;       // the caches again, writable
   half_t* vcache_w;
+  uint8_t* real_w;        // the mask again, writable: the new token's position becomes real
   float eps, clip;
   int max_positions;
 };
@@ -439,6 +447,8 @@ decode_attention_kernel(const half_t* __restrict__ q, const half_t* kcache, cons
       const size_t at = (((size_t)b * kv_heads + kvh) * capacity + slot) * D + c * 8;
       *reinterpret_cast<half8_t*>(nt.kcache_w + at) = knew;
       *reinterpret_cast<half8_t*>(nt.vcache_w + at) = vnew;
+      // no workgroup of this launch reads the mask at `slot`: the loop stops before it
+      if (qh == 0 && c == 0) nt.real_w[(size_t)b * capacity + slot] = 1;
     }
   } else {
     const half8_t qv = *reinterpret_cast<const half8_t*>(q + ((size_t)b * heads + qh) * D + c * 8);
@@ -484,7 +494,7 @@ decode_attention_kernel(const half_t* __restrict__ q, const half_t* kcache, cons
 #pragma unroll
     for (int j = 0; j < 8; ++j) d += qf[j] * (float)knew[j];
     const float sc = key_sum<LPK>(d);
-    const bool ok = sub == 0 && rl[slot] != 0;
+    const bool ok = sub == 0;   // the new token is real
     const float mx = ok ? fmaxf(m, sc) : m;
     const float alpha = __builtin_amdgcn_exp2f(m - mx);
     const float p = ok ? __builtin_amdgcn_exp2f(sc - mx) : 0.f;
@@ -532,6 +542,69 @@ decode_attention_kernel(const half_t* __restrict__ q, const half_t* kcache, cons
   }
 }
 
+// One workgroup per sequence: the arg-max of its logits (the lowest index among equal maxima)
+// becomes its next token, is appended to its output row, and its rotary position advances;
+// the first workgroup also advances the cache slot, which nothing in this launch reads.
+constexpr int PICK_THREADS = 1024;
+
+__global__ void __launch_bounds__(PICK_THREADS)
+greedy_advance_kernel(const half_t* __restrict__ logits, int V, int64_t* __restrict__ tok, int64_t* __restrict__ out,
+                      int out_stride, const int64_t* __restrict__ base_position, int64_t* __restrict__ next_position,
+                      int64_t* __restrict__ slot) {
+  __shared__ float best_v[PICK_THREADS / WAVE];
+  __shared__ int best_i[PICK_THREADS / WAVE];
+  const int b = blockIdx.x, tid = threadIdx.x;
+  const half_t* row = logits + (size_t)b * V;
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  const int chunks = V % 8 == 0 ? V >> 3 : 0;   // 16-byte loads need rows that start on 16 bytes
+  for (int c = tid; c < chunks; c += PICK_THREADS) {
+    const half8_t v = *reinterpret_cast<const half8_t*>(row + c * 8);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float f = (float)v[j];
+      if (f > bv) {           // ascending indices per thread: the first of equal values is kept
+        bv = f;
+        bi = c * 8 + j;
+      }
+    }
+  }
+  for (int i = chunks * 8 + tid; i < V; i += PICK_THREADS) {
+    const float f = (float)row[i];
+    if (f > bv) {
+      bv = f;
+      bi = i;
+    }
+  }
+  // wavefront, then workgroup: larger value wins, equal values go to the lower index
+  for (int off = 32; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(bv, off, WAVE);
+    const int oi = __shfl_xor(bi, off, WAVE);
+    if (ov > bv || (ov == bv && oi < bi)) {
+      bv = ov;
+      bi = oi;
+    }
+  }
+  if ((tid & 63) == 0) {
+    best_v[tid >> 6] = bv;
+    best_i[tid >> 6] = bi;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    for (int w = 1; w < PICK_THREADS / WAVE; ++w)
+      if (best_v[w] > bv || (best_v[w] == bv && best_i[w] < bi)) {
+        bv = best_v[w];
+        bi = best_i[w];
+      }
+    if (bi == 0x7fffffff) bi = 0;   // a row of NaNs or -inf: token 0
+    tok[b] = bi;
+    const long col = (long)(next_position[b] - base_position[b]);
+    if (col >= 0 && col < out_stride) out[(size_t)b * out_stride + col] = bi;
+    next_position[b] += 1;
+    if (b == 0) *slot += 1;
+  }
+}
+
 }  // namespace
 
 #define ROW_LIMITS(what)                                                                          \
@@ -545,8 +618,20 @@ extern "C" SY_API int sy_add_rmsnorm(const void* x, const void* delta, const voi
   SY_REQUIRE(x && weight && h_out, "add_rmsnorm: null pointer");
   row_kernel<false, false><<<N, ROW_THREADS, 0, (hipStream_t)stream>>>(
       (const half_t*)x, (const half_t*)delta, nullptr, nullptr, nullptr, 0, (const half_t*)weight, eps, nullptr, 0, H,
-      (half_t*)x_out, (half_t*)h_out, nullptr);
+      (half_t*)x_out, (half_t*)h_out, nullptr, nullptr, 0);
   return sy_check_launch("add_rmsnorm");
+}
+
+extern "C" SY_API int sy_embed_rmsnorm(const int64_t* tokens, const void* embed, int vocab, const void* weight, float eps,
+                                       int N, int H, void* x_out, void* h_out, void* stream) {
+  ROW_LIMITS("embed_rmsnorm");
+  SY_REQUIRE(vocab >= 1, "embed_rmsnorm: vocab = %d", vocab);
+  if (N == 0) return SY_OK;
+  SY_REQUIRE(tokens && embed && weight && x_out && h_out, "embed_rmsnorm: null pointer");
+  row_kernel<false, false><<<N, ROW_THREADS, 0, (hipStream_t)stream>>>(
+      (const half_t*)embed, nullptr, nullptr, nullptr, nullptr, 0, (const half_t*)weight, eps, nullptr, 0, H,
+      (half_t*)x_out, (half_t*)h_out, nullptr, tokens, vocab);
+  return sy_check_launch("embed_rmsnorm");
 }
 
 extern "C" SY_API int sy_add_rmsnorm_logits(const void* x, const void* delta, const void* weight, float eps,
@@ -558,7 +643,7 @@ extern "C" SY_API int sy_add_rmsnorm_logits(const void* x, const void* delta, co
   SY_REQUIRE(x && weight && h_out && router && logits, "add_rmsnorm_logits: null pointer");
   row_kernel<false, true><<<N, 1024, (size_t)H * sizeof(half_t), (hipStream_t)stream>>>(
       (const half_t*)x, (const half_t*)delta, nullptr, nullptr, nullptr, 0, (const half_t*)weight, eps,
-      (const half_t*)router, E, H, (half_t*)x_out, (half_t*)h_out, (half_t*)logits);
+      (const half_t*)router, E, H, (half_t*)x_out, (half_t*)h_out, (half_t*)logits, nullptr, 0);
   return sy_check_launch("add_rmsnorm_logits");
 }
 
@@ -571,7 +656,7 @@ extern "C" SY_API int sy_combine_add_rmsnorm(const void* y, const int32_t* pos_o
   SY_REQUIRE(y && pos_of && idx && x && weight && h_out, "combine_add_rmsnorm: null pointer");
   row_kernel<true, false><<<N, ROW_THREADS, 0, (hipStream_t)stream>>>(
       (const half_t*)x, nullptr, (const half_t*)y, pos_of, idx, k, (const half_t*)weight, eps, nullptr, 0, H,
-      (half_t*)x_out, (half_t*)h_out, nullptr);
+      (half_t*)x_out, (half_t*)h_out, nullptr, nullptr, 0);
   return sy_check_launch("combine_add_rmsnorm");
 }
 
@@ -622,7 +707,7 @@ extern "C" SY_API int sy_decode_attention(const void* q, const void* kcache, con
 
 extern "C" SY_API int sy_decode_attention_qkv(const void* qkv, const void* q_norm, const void* k_norm, float eps, float clip,
                                               const void* cos_table, const void* sin_table, int max_positions,
-                                              const int64_t* positions, const int64_t* slot, const uint8_t* real, int B,
+                                              const int64_t* positions, const int64_t* slot, uint8_t* real, int B,
                                               int heads, int kv_heads, int D, int capacity, void* kcache, void* vcache,
                                               void* out, void* stream) {
   SY_REQUIRE(B >= 0 && heads >= 1 && kv_heads >= 1 && heads % kv_heads == 0,
@@ -638,11 +723,22 @@ extern "C" SY_API int sy_decode_attention_qkv(const void* qkv, const void* q_nor
   const size_t lds = (size_t)waves * (D + 2) * sizeof(float);
   const float scale_log2e = 1.4426950408889634f / sqrtf((float)D);
   NewToken nt{(const half_t*)qkv, (const half_t*)q_norm, (const half_t*)k_norm, (const half_t*)cos_table,
-              (const half_t*)sin_table, positions, (half_t*)kcache, (half_t*)vcache, eps, clip, max_positions};
+              (const half_t*)sin_table, positions, (half_t*)kcache, (half_t*)vcache, real, eps, clip, max_positions};
   auto kern = D == 128 ? (waves == 4 ? decode_attention_kernel<16, true, 4, 4> : decode_attention_kernel<16, true, 16, 4>)
                        : (waves == 4 ? decode_attention_kernel<8, true, 4, 4> : decode_attention_kernel<8, true, 16, 4>);
   kern<<<(unsigned)pairs, waves * WAVE, lds, (hipStream_t)stream>>>(nullptr, (const half_t*)kcache, (const half_t*)vcache,
                                                                    real, slot, heads, kv_heads, capacity, scale_log2e,
                                                                    (half_t*)out, nt);
   return sy_check_launch("decode_attention_qkv");
+}
+
+extern "C" SY_API int sy_greedy_advance(const void* logits, int B, int V, int64_t* tok, int64_t* out, int out_stride,
+                                        const int64_t* base_position, int64_t* next_position, int64_t* slot,
+                                        void* stream) {
+  SY_REQUIRE(B >= 0 && V >= 1 && out_stride >= 0, "greedy_advance: B = %d, V = %d, out_stride = %d", B, V, out_stride);
+  if (B == 0) return SY_OK;
+  SY_REQUIRE(logits && tok && out && base_position && next_position && slot, "greedy_advance: null pointer");
+  greedy_advance_kernel<<<B, PICK_THREADS, 0, (hipStream_t)stream>>>((const half_t*)logits, V, tok, out, out_stride,
+                                                                    base_position, next_position, slot);
+  return sy_check_launch("greedy_advance");
 }

@@ -259,19 +259,19 @@ class Decoder:
         return self._wqkv
 
     @torch.no_grad()
-    def step_fused(self, tok, cache, slot, keys=None):
-        """The same step as `step_static` on the decode kernels: residual add + RMS norm, the
+    def step_fused(self, tok, cache, slot, keys=None, advance=True):
+        """The same step as `step_static` on the decode kernels: embedding + RMS norm, the
         stacked q/k/v projection, attention over the cache (with the q/k norm, the rotary
-        embedding and the cache write in its prologue), the output projection, and the MoE
-        hook; every projection streams its weights once."""
+        embedding and the cache write in its prologue), the output projection, residual add +
+        RMS norm, and the MoE hook; every projection streams its weights once. With
+        advance=False the cache counters are left to the caller (`greedy_advance` moves them
+        together with the arg-max)."""
         from . import kernels
 
         s, W, E = self.s, self.w, kernels.ext()
         wqkv = self._stacked_qkv()
         positions = cache.next_position
-        cache.real.index_fill_(1, slot, True)
-        x = F.embedding(tok[:, 0], W["embed"])
-        x, xn = E.add_rmsnorm(x, None, W["layers"][0]["attn_norm"], s.rms_eps)
+        x, xn = E.embed_rmsnorm(tok.reshape(-1), W["embed"], W["layers"][0]["attn_norm"], s.rms_eps)
         for i in range(s.layers):
             L = W["layers"][i]
             after = W["layers"][i + 1]["attn_norm"] if i + 1 < s.layers else W["final_norm"]
@@ -287,8 +287,9 @@ class Decoder:
             else:
                 x, h = E.add_rmsnorm(x, o, L["mlp_norm"], s.rms_eps, x_out=x)
                 x, xn = E.add_rmsnorm(x, self.moe(i, h), after, s.rms_eps, x_out=x)
-        cache.next_position += 1
-        slot += 1
+        if advance:
+            cache.next_position += 1
+            slot += 1
         return kernels.dense(xn, W["lm_head"])
 
     def step(self, tok, cache, slot, keys):
@@ -327,26 +328,34 @@ class Decoder:
             col = torch.ones(1, dtype=torch.long, device=dev)       # column of `out` the next token goes to
             keys = torch.arange(cache.capacity, device=dev)
 
-            def one_token():
-                logits = self.step(tok, cache, slot, keys)
-                tok.copy_(logits.argmax(-1)[:, None])
-                out.index_copy_(1, col, tok)
-                col.add_(1)
+            if self.fused:
+                from . import kernels
+                base = cache.next_position - 1          # column 1 of `out` is due now
+
+                def one_token():
+                    logits = self.step_fused(tok, cache, slot, advance=False)
+                    kernels.ext().greedy_advance(logits, tok, out, base, cache.next_position, slot)
+            else:
+                def one_token():
+                    logits = self.step_static(tok, cache, slot, keys)
+                    tok.copy_(logits.argmax(-1)[:, None])
+                    out.index_copy_(1, col, tok)
+                    col.add_(1)
 
             # warm up on a side stream (allocator, kernel loading), then restore the state it touched
-            saved = (cache.next_position.clone(), slot.clone(), col.clone(), tok.clone(), cache.real.clone())
+            saved = (cache.next_position.clone(), slot.clone(), col.clone(), tok.clone(), cache.real.clone(), out.clone())
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(side):
                 one_token()
             torch.cuda.current_stream().wait_stream(side)
             cache.next_position.copy_(saved[0]); slot.copy_(saved[1]); col.copy_(saved[2]); tok.copy_(saved[3])
-            cache.real.copy_(saved[4])
+            cache.real.copy_(saved[4]); out.copy_(saved[5])
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 one_token()
             cache.next_position.copy_(saved[0]); slot.copy_(saved[1]); col.copy_(saved[2]); tok.copy_(saved[3])
-            cache.real.copy_(saved[4])
+            cache.real.copy_(saved[4]); out.copy_(saved[5])
             if timings is not None:
                 torch.cuda.synchronize()
                 t0 = time.perf_counter()
@@ -375,23 +384,37 @@ class Decoder:
         cache = KVCache(self.s, B, P + max_new_tokens, dtype, dev)
         logits = self.forward(tokens, cache, valid)[:, -1]
         first_logits = logits
-        out = torch.empty(B, max_new_tokens, dtype=torch.long, device=dev)
+        out = torch.zeros(B, max_new_tokens, dtype=torch.long, device=dev)
         steps = 0
         alive = torch.ones(B, dtype=torch.bool, device=dev)
-        slot = torch.tensor([cache.filled], dtype=torch.long, device=dev) if self.fused else None
-        for step in range(max_new_tokens):
-            nxt = logits.argmax(-1)
-            out[:, step] = nxt
-            steps = step + 1
-            if eos is not None:
-                alive &= nxt != eos
-                if not bool(alive.any()):
-                    break
-            if step + 1 < max_new_tokens:
-                if self.fused:   # the launches `generate_graph` replays, issued one by one
-                    logits = self.step_fused(nxt[:, None], cache, slot)
-                    cache.filled += 1
-                else:
+        if self.fused:
+            # the launches `generate_graph` replays, issued one by one: the step on the decode
+            # kernels, then arg-max, append and counters in one launch
+            from . import kernels
+            tok = logits.argmax(-1)[:, None].clone()
+            out[:, 0] = tok[:, 0]
+            steps = 1
+            slot = torch.tensor([cache.filled], dtype=torch.long, device=dev)
+            base = cache.next_position - 1
+            for step in range(1, max_new_tokens):
+                if eos is not None:
+                    alive &= tok[:, 0] != eos
+                    if not bool(alive.any()):
+                        break
+                step_logits = self.step_fused(tok, cache, slot, advance=False)
+                kernels.ext().greedy_advance(step_logits, tok, out, base, cache.next_position, slot)
+                cache.filled += 1
+                steps = step + 1
+        else:
+            for step in range(max_new_tokens):
+                nxt = logits.argmax(-1)
+                out[:, step] = nxt
+                steps = step + 1
+                if eos is not None:
+                    alive &= nxt != eos
+                    if not bool(alive.any()):
+                        break
+                if step + 1 < max_new_tokens:
                     logits = self.forward(nxt[:, None], cache)[:, -1]
         rows = out[:, :steps].tolist()
         if eos is not None:

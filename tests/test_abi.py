@@ -26,7 +26,8 @@ def declared_symbols(header=None):
 
 def test_header_declares_the_expected_entry_points():
     assert sorted(declared_symbols(DECODE_HEADER)) == ["sy_add_rmsnorm", "sy_add_rmsnorm_logits", "sy_combine_add_rmsnorm",
-                                                       "sy_decode_attention", "sy_decode_attention_qkv", "sy_qk_norm_rope_cache"]
+                                                       "sy_decode_attention", "sy_decode_attention_qkv", "sy_embed_rmsnorm",
+                                                       "sy_greedy_advance", "sy_qk_norm_rope_cache"]
     assert sorted(os.listdir(os.path.join(ROOT, "include"))) == ["switchyard_decode.h", "switchyard_moe.h"]
     assert sorted(declared_symbols(HEADER)) == sorted(["sy_version", "sy_last_error", "sy_route", "sy_sort_workspace_bytes",
                                                   "sy_sort_by_expert", "sy_route_sort",
@@ -61,6 +62,11 @@ def test_decode_argument_errors_and_empty_batches(lib):
     assert b"multiple of 8" in lib.sy_last_error()
     assert lib.sy_add_rmsnorm(None, None, None, 1e-5, 4, 16384, None, None, None) == 1
     assert lib.sy_add_rmsnorm(None, None, None, 1e-5, 0, 2048, None, None, None) == 0
+    assert lib.sy_embed_rmsnorm(None, None, 0, None, 1e-5, 4, 2048, None, None, None) == 1
+    assert lib.sy_embed_rmsnorm(None, None, 100, None, 1e-5, 0, 2048, None, None, None) == 0
+    assert lib.sy_greedy_advance(None, 4, 0, None, None, 8, None, None, None, None) == 1
+    assert lib.sy_greedy_advance(None, 0, 1000, None, None, 8, None, None, None, None) == 0
+    assert lib.sy_greedy_advance(None, 4, 1000, None, None, 8, None, None, None, None) == 1   # null pointers
     assert lib.sy_add_rmsnorm_logits(None, None, None, 1e-5, None, 2000, 4, 2048, None, None, None, None) == 1
     assert lib.sy_add_rmsnorm_logits(None, None, None, 1e-5, None, 64, 0, 2048, None, None, None, None) == 0
     assert lib.sy_combine_add_rmsnorm(None, None, None, 65, None, None, 1e-5, 4, 2048, None, None, None) == 1

@@ -77,6 +77,49 @@ def test_combine_add_rmsnorm(N, H, E, k):
     assert xo3 is x3 and torch.equal(x3, xo) and torch.equal(h3, h)
 
 
+@pytest.mark.parametrize("N,H,vocab", [(8, 2048, 50304), (64, 2048, 50304), (3, 64, 10), (1, 520, 77)])
+def test_embed_rmsnorm(N, H, vocab):
+    """The embedding rows bit for bit, their norm as add_rmsnorm gives it; ids outside the table are clamped."""
+    g = torch.Generator().manual_seed(1)
+    embed, w = rnd(vocab, H, seed=2), 1 + rnd(H, seed=3, std=0.1)
+    tokens = torch.randint(0, vocab, (N,), generator=g).cuda()
+    x, h = kernels.ext().embed_rmsnorm(tokens, embed, w, 1e-5)
+    assert torch.equal(x, embed[tokens])
+    assert torch.equal(h, kernels.ext().add_rmsnorm(embed[tokens].contiguous(), None, w, 1e-5)[1])
+    wild = tokens.clone()
+    wild[0] = vocab + 5
+    x2, _ = kernels.ext().embed_rmsnorm(wild, embed, w, 1e-5)
+    assert torch.equal(x2[0], embed[vocab - 1])
+
+
+@pytest.mark.parametrize("B,V", [(8, 50304), (64, 50304), (3, 1000), (2, 131), (1, 8)])
+def test_greedy_advance(B, V):
+    """Arg-max with the lowest index among equal maxima, the token appended at the column the
+    sequence's position names, the counters advanced; twice in a row."""
+    g = torch.Generator().manual_seed(4)
+    ext = kernels.ext()
+    tok = torch.zeros(B, 1, dtype=torch.long, device="cuda")
+    out = torch.full((B, 5), -1, dtype=torch.long, device="cuda")
+    nxt = torch.randint(5, 50, (B,), generator=g).cuda()
+    base = nxt - 2                      # column 2 is due
+    start = nxt.clone()
+    slot = torch.tensor([17], device="cuda")
+    for call in range(2):
+        logits = (torch.randn(B, V, generator=g) * 3).half()
+        top = logits.max(-1).values
+        logits[0, V // 2] = top[0]      # a tie, possibly above the first maximum's index
+        logits[-1, 0] = logits[-1].max()
+        want = torch.tensor([int(torch.where(r == r.max())[0][0]) for r in logits])
+        ext.greedy_advance(logits.cuda(), tok, out, base, nxt, slot)
+        assert torch.equal(tok[:, 0].cpu(), want)
+        assert torch.equal(out[:, 2 + call].cpu(), want) and int((out[:, 4] != -1).sum()) == 0
+        assert torch.equal(nxt, start + call + 1) and int(slot) == 18 + call
+    assert int((out[:, :2] != -1).sum()) == 0
+    # a column outside the output is not written
+    ext.greedy_advance(logits.cuda(), tok, out, nxt + 1, nxt, slot)
+    assert int((out[:, 4] != -1).sum()) == 0
+
+
 def torch_qk_step(qkv, L, s, cos, sin, positions, clip):
     """q, k (normed, clamped, rotated) and v of one new token, as Decoder.step_static does."""
     B = qkv.shape[0]
@@ -176,15 +219,18 @@ def test_attention_with_the_norm_and_rotary_in_its_prologue(B, heads, kv_heads, 
     ext = kernels.ext()
     q = ext.qk_norm_rope_cache(qkv, qn, kn, s.rms_eps, clip, dec.cos, dec.sin, positions, slot, heads, kv_heads, hd, kc, vc)
     want = ext.decode_attention(q, kc, vc, real, slot, heads)
-    got = ext.decode_attention_qkv(qkv, qn, kn, s.rms_eps, clip, dec.cos, dec.sin, positions, slot, real, heads, kv_heads,
-                                   hd, kc2, vc2)
+    unmarked = real.clone()
+    unmarked[:, slot_at] = False          # the launch itself declares the new token real
+    got = ext.decode_attention_qkv(qkv, qn, kn, s.rms_eps, clip, dec.cos, dec.sin, positions, slot, unmarked, heads,
+                                   kv_heads, hd, kc2, vc2)
+    assert torch.equal(unmarked, real)
     assert torch.equal(kc2, kc) and torch.equal(vc2, vc)
     assert torch.allclose(got.float(), want.float(), rtol=2 * ULP, atol=1e-3)
     # a slot past the cache: nothing is written, every cached key is visible
     slot_out = torch.tensor([cap], device="cuda")
-    got = ext.decode_attention_qkv(qkv, qn, kn, s.rms_eps, clip, dec.cos, dec.sin, positions, slot_out, real, heads,
+    got = ext.decode_attention_qkv(qkv, qn, kn, s.rms_eps, clip, dec.cos, dec.sin, positions, slot_out, unmarked, heads,
                                    kv_heads, hd, kc2, vc2)
-    assert torch.equal(kc2, kc) and torch.equal(vc2, vc)
+    assert torch.equal(kc2, kc) and torch.equal(vc2, vc) and torch.equal(unmarked, real)
     want = ext.decode_attention(q, kc, vc, real, slot_out, heads)
     assert torch.allclose(got.float(), want.float(), rtol=2 * ULP, atol=1e-3)
 
