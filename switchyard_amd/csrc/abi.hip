@@ -35,6 +35,6 @@ int sy_compute_units() {
   return cached[dev];
 }
 
-extern "C" SY_API int sy_version(void) { return 100; }
+extern "C" SY_API int sy_version(void) { return 200; }  // 0.2.0: the decode-step entry points
 
 extern "C" SY_API const char* sy_last_error(void) { return g_error; }
