@@ -52,22 +52,22 @@ SY_API int sy_add_rmsnorm_logits(const void* x, const void* delta, const void* w
 SY_API int sy_combine_add_rmsnorm(const void* y, const int32_t* pos_of, const int32_t* idx, int k, const void* x,
                                   const void* weight, float eps, int N, int H, void* x_out, void* h_out, void* stream);
 
-/* What follows the q/k/v projections of one new token per sequence; replaces the rmsnorm of q
- * and k, the clamp, the rotary embedding and the cache write of _attention()
- * (switchyard/model.py:64-77) with T = 1.
- * qkv f16 [B, (heads + 2*kv_heads)*D]: a row holds q, then k, then v; q_norm f16 [heads*D],
- * k_norm f16 [kv_heads*D] (the norm runs over the whole projection, not per head);
- * clip > 0 clamps q, k and v to [-clip, clip]; cos_table, sin_table f16 [max_positions, D]
- * (both halves of a row equal, as cat([freqs, freqs])); positions int64 [B] rotary position of
- * each sequence's new token; slot int64 [1] cache position to write (the same for every
- * sequence of a left-padded batch) ->
- * q_out f16 [B, heads*D]; kcache, vcache f16 [B, kv_heads, capacity, D] get the new key and
- * value at [:, :, slot, :]. A slot outside [0, capacity) writes nothing.
+/* What follows the q/k/v projections of T new tokens per sequence (T = 1 at decode, the prompt
+ * length at prefill); replaces the rmsnorm of q and k, the clamp, the rotary embedding and the
+ * cache write of _attention() (switchyard/model.py:64-77).
+ * qkv f16 [B*T, (heads + 2*kv_heads)*D]: row b*T + t holds q, then k, then v of token t of
+ * sequence b; q_norm f16 [heads*D], k_norm f16 [kv_heads*D] (the norm runs over the whole
+ * projection, not per head); clip > 0 clamps q, k and v to [-clip, clip]; cos_table, sin_table
+ * f16 [max_positions, D] (both halves of a row equal, as cat([freqs, freqs])); positions int64
+ * [B*T] rotary position of each token; slot int64 [1] cache position of token 0 (the same for
+ * every sequence of a left-padded batch) ->
+ * q_out f16 [B*T, heads*D]; kcache, vcache f16 [B, kv_heads, capacity, D] get the new keys and
+ * values at [:, :, slot + t, :]. A position outside [0, capacity) is not written.
  * Limits: D % 16 == 0, heads*D <= 8192, heads % kv_heads == 0. B == 0 is a no-op. */
 SY_API int sy_qk_norm_rope_cache(const void* qkv, const void* q_norm, const void* k_norm, float eps, float clip,
                                  const void* cos_table, const void* sin_table, int max_positions,
-                                 const int64_t* positions, const int64_t* slot, int B, int heads, int kv_heads, int D,
-                                 int capacity, void* q_out, void* kcache, void* vcache, void* stream);
+                                 const int64_t* positions, const int64_t* slot, int B, int T, int heads, int kv_heads,
+                                 int D, int capacity, void* q_out, void* kcache, void* vcache, void* stream);
 
 /* One query per (sequence, head) against the KV cache; replaces the scores / mask / softmax /
  * value product of _attention() (switchyard/model.py:78-84) with T = 1.

@@ -45,7 +45,7 @@ SIGNATURES = {
     "sy_combine_add_rmsnorm": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_float, _c_int,
                                         _c_int, _c_void_p, _c_void_p, _c_void_p]),
     "sy_qk_norm_rope_cache": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_float, _c_void_p, _c_void_p, _c_int,
-                                       _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p,
+                                       _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p,
                                        _c_void_p, _c_void_p, _c_void_p]),
     "sy_decode_attention_qkv": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_float, _c_void_p, _c_void_p, _c_int,
                                          _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int,
@@ -277,28 +277,30 @@ class Ext:
 
     def qk_norm_rope_cache(self, qkv, q_norm, k_norm, eps, clip, cos, sin, positions, slot, heads, kv_heads, head_dim,
                            kcache, vcache):
-        """qkv [B, (heads + 2 kv_heads) D] -> q [B, heads D] normed and rotated; the new key and
-        value go into kcache / vcache [B, kv_heads, capacity, D] at the device-held `slot`."""
+        """qkv [B*T, (heads + 2 kv_heads) D] (T tokens per sequence, T = rows / batch of the caches)
+        -> q [B*T, heads D] normed and rotated; the new keys and values go into kcache / vcache
+        [B, kv_heads, capacity, D] from the device-held `slot` on."""
         for t, name in ((qkv, "qkv"), (q_norm, "q_norm"), (k_norm, "k_norm"), (cos, "cos"), (sin, "sin"),
                         (kcache, "kcache"), (vcache, "vcache")):
             _check(t, name, torch.float16)
         _check(positions, "positions", torch.int64)
         _check(slot, "slot", torch.int64)
-        B, D = qkv.shape[0], int(head_dim)
+        rows, D = qkv.shape[0], int(head_dim)
         if qkv.shape[1] != (heads + 2 * kv_heads) * D or q_norm.numel() != heads * D or k_norm.numel() != kv_heads * D:
             raise RuntimeError("qk_norm_rope_cache: qkv / q_norm / k_norm do not match heads, kv_heads and head_dim")
         if cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] != D:
             raise RuntimeError("qk_norm_rope_cache: cos and sin must be [max_positions, head_dim]")
-        if kcache.shape != vcache.shape or kcache.dim() != 4 or tuple(kcache.shape[:2]) != (B, kv_heads) or \
-                kcache.shape[3] != D:
+        if kcache.shape != vcache.shape or kcache.dim() != 4 or kcache.shape[1] != kv_heads or kcache.shape[3] != D:
             raise RuntimeError("qk_norm_rope_cache: caches must be [B, kv_heads, capacity, head_dim]")
-        if positions.numel() != B or slot.numel() != 1:
-            raise RuntimeError("qk_norm_rope_cache: positions [B] and slot [1]")
-        q = torch.empty((B, heads * D), dtype=torch.float16, device=qkv.device)
+        B = kcache.shape[0]
+        if B == 0 or rows % B or positions.numel() != rows or slot.numel() != 1:
+            raise RuntimeError("qk_norm_rope_cache: qkv needs T rows per sequence of the caches, positions one entry "
+                               "per row, slot one entry")
+        q = torch.empty((rows, heads * D), dtype=torch.float16, device=qkv.device)
         self._call(self.lib.sy_qk_norm_rope_cache, qkv.data_ptr(), q_norm.data_ptr(), k_norm.data_ptr(), float(eps),
                    float(clip or 0.0), cos.data_ptr(), sin.data_ptr(), cos.shape[0], positions.data_ptr(),
-                   slot.data_ptr(), B, int(heads), int(kv_heads), D, kcache.shape[2], q.data_ptr(), kcache.data_ptr(),
-                   vcache.data_ptr(), _stream())
+                   slot.data_ptr(), B, rows // B, int(heads), int(kv_heads), D, kcache.shape[2], q.data_ptr(),
+                   kcache.data_ptr(), vcache.data_ptr(), _stream())
         return q
 
     def decode_attention(self, q, kcache, vcache, real, slot, heads):

@@ -190,21 +190,22 @@ __device__ __forceinline__ half_t rotary_f16(half_t y, half_t rot, half_t cos_v,
   return (half_t)((float)t1 + (float)t2);
 }
 
-// One workgroup per sequence. qkv row = [q (heads*D) | k (kv_heads*D) | v (kv_heads*D)].
+// One workgroup per token. qkv row = [q (heads*D) | k (kv_heads*D) | v (kv_heads*D)].
 __global__ void __launch_bounds__(ROW_THREADS)
 qk_norm_rope_cache_kernel(const half_t* __restrict__ qkv, const half_t* __restrict__ q_norm,
                           const half_t* __restrict__ k_norm, float eps, float clip, const half_t* __restrict__ cos_t,
                           const half_t* __restrict__ sin_t, int max_positions, const int64_t* __restrict__ positions,
-                          const int64_t* __restrict__ slot_ptr, int heads, int kv_heads, int D, int capacity,
+                          const int64_t* __restrict__ slot_ptr, int T, int heads, int kv_heads, int D, int capacity,
                           half_t* __restrict__ q_out, half_t* __restrict__ kcache, half_t* __restrict__ vcache) {
   extern __shared__ __attribute__((aligned(16))) half_t normed[];  // [qd + kvd] after norm and clamp
   __shared__ float part[32];
-  const int b = blockIdx.x;
+  // row r of qkv is token t = r % T of sequence b = r / T; it goes to cache position slot + t
+  const int r = blockIdx.x, b = r / T;
   const int qd = heads * D, kvd = kv_heads * D;
-  const half_t* row = qkv + (size_t)b * (qd + 2 * kvd);
+  const half_t* row = qkv + (size_t)r * (qd + 2 * kvd);
   const int qchunks = qd >> 3, kchunks = kvd >> 3;
-  const long slot = (long)*slot_ptr;
-  long pos = (long)positions[b];
+  const long slot = (long)*slot_ptr + (r - b * T);
+  long pos = (long)positions[r];
   pos = pos < 0 ? 0 : pos >= max_positions ? max_positions - 1 : pos;
   const bool slot_ok = slot >= 0 && slot < capacity;
 
@@ -266,7 +267,7 @@ qk_norm_rope_cache_kernel(const half_t* __restrict__ qkv, const half_t* __restri
       o[j] = rotary_f16(y[j], low ? -other[j] : other[j], cc[j], ssn[j]);
     }
     if (c < qchunks) {
-      *reinterpret_cast<half8_t*>(q_out + (size_t)b * qd + c * 8) = o;
+      *reinterpret_cast<half8_t*>(q_out + (size_t)r * qd + c * 8) = o;
     } else if (slot_ok) {
       const int e = (c - qchunks) * 8, h = e / D;
       *reinterpret_cast<half8_t*>(kcache + (((size_t)b * kv_heads + h) * capacity + slot) * D + (e - h * D)) = o;
@@ -662,11 +663,11 @@ extern "C" SY_API int sy_combine_add_rmsnorm(const void* y, const int32_t* pos_o
 
 extern "C" SY_API int sy_qk_norm_rope_cache(const void* qkv, const void* q_norm, const void* k_norm, float eps, float clip,
                                             const void* cos_table, const void* sin_table, int max_positions,
-                                            const int64_t* positions, const int64_t* slot, int B, int heads,
+                                            const int64_t* positions, const int64_t* slot, int B, int T, int heads,
                                             int kv_heads, int D, int capacity, void* q_out, void* kcache, void* vcache,
                                             void* stream) {
-  SY_REQUIRE(B >= 0 && heads >= 1 && kv_heads >= 1 && heads % kv_heads == 0,
-             "qk_norm_rope_cache: B = %d, heads = %d, kv_heads = %d", B, heads, kv_heads);
+  SY_REQUIRE(B >= 0 && T >= 1 && (long)B * T < (1l << 31) && heads >= 1 && kv_heads >= 1 && heads % kv_heads == 0,
+             "qk_norm_rope_cache: B = %d, T = %d, heads = %d, kv_heads = %d", B, T, heads, kv_heads);
   SY_REQUIRE(D >= 16 && D % 16 == 0 && (long)heads * D <= 8 * ROW_THREADS * MAX_CHUNKS,
              "qk_norm_rope_cache: head_dim = %d must be a multiple of 16 and heads * head_dim at most %d", D,
              8 * ROW_THREADS * MAX_CHUNKS);
@@ -676,9 +677,9 @@ extern "C" SY_API int sy_qk_norm_rope_cache(const void* qkv, const void* q_norm,
   SY_REQUIRE(qkv && q_norm && k_norm && cos_table && sin_table && positions && slot && q_out && kcache && vcache,
              "qk_norm_rope_cache: null pointer");
   const size_t lds = (size_t)(heads + kv_heads) * D * sizeof(half_t);
-  qk_norm_rope_cache_kernel<<<B, ROW_THREADS, lds, (hipStream_t)stream>>>(
+  qk_norm_rope_cache_kernel<<<B * T, ROW_THREADS, lds, (hipStream_t)stream>>>(
       (const half_t*)qkv, (const half_t*)q_norm, (const half_t*)k_norm, eps, clip, (const half_t*)cos_table,
-      (const half_t*)sin_table, max_positions, positions, slot, heads, kv_heads, D, capacity, (half_t*)q_out,
+      (const half_t*)sin_table, max_positions, positions, slot, T, heads, kv_heads, D, capacity, (half_t*)q_out,
       (half_t*)kcache, (half_t*)vcache);
   return sy_check_launch("qk_norm_rope_cache");
 }

@@ -172,11 +172,8 @@ class Decoder:
         a = F.scaled_dot_product_attention(q, k, v, attn_mask=mask, enable_gqa=s.kv_heads != s.heads)
         return F.linear(a.transpose(1, 2).reshape(B, T, s.heads * s.head_dim), L["wo"])
 
-    @torch.no_grad()
-    def forward(self, tokens, cache=None, valid=None):
-        """tokens [B, T] -> logits [B, T, vocab]. `valid` [B, T] marks real tokens (False = left
-        padding). With a cache the tokens are appended after what it already holds."""
-        s, W = self.s, self.w
+    def _prepare(self, tokens, cache, valid):
+        """Rotary positions and the attention mask of `tokens` [B, T] appended to `cache`."""
         B, T = tokens.shape
         dev = tokens.device
         if valid is None:
@@ -195,8 +192,15 @@ class Decoder:
         kj = torch.arange(start + T, device=dev)[None, :]
         mask = (kj <= qi)[None] & keys_real[:, None, :]
         mask = mask | ((kj == qi)[None] & ~mask.any(-1, keepdim=True))
-        mask = mask[:, None]  # broadcast over heads
+        return valid, start, base, positions, mask[:, None]  # the mask broadcasts over heads
 
+    @torch.no_grad()
+    def forward(self, tokens, cache=None, valid=None):
+        """tokens [B, T] -> logits [B, T, vocab]. `valid` [B, T] marks real tokens (False = left
+        padding). With a cache the tokens are appended after what it already holds."""
+        s, W = self.s, self.w
+        B, T = tokens.shape
+        valid, start, base, positions, mask = self._prepare(tokens, cache, valid)
         x = F.embedding(tokens, W["embed"])
         for i in range(s.layers):
             L = W["layers"][i]
@@ -207,6 +211,49 @@ class Decoder:
             cache.filled = start + T
             cache.next_position = base + valid.long().sum(1)
         return F.linear(_rms(x, W["final_norm"], s.rms_eps), W["lm_head"])
+
+    @torch.no_grad()
+    def prefill_fused(self, tokens, cache, valid=None):
+        """`forward` for a prompt on the library's kernels, returning the logits of the last
+        position only, [B, vocab]: norms, residual adds, the q/k norm with the rotary embedding
+        and the cache write are one launch each over all B*T rows (in PyTorch they are some
+        seventy element-wise launches per layer, each a pass over the activations), the three
+        input projections are one GEMM, and the lm_head runs on B rows instead of B*T.
+        Attention itself is PyTorch's fused scaled-dot-product call under the same mask."""
+        from . import kernels
+
+        s, W, E = self.s, self.w, kernels.ext()
+        B, T = tokens.shape
+        valid, start, base, positions, mask = self._prepare(tokens, cache, valid)
+        wqkv = self._stacked_qkv()
+        slot = torch.tensor([start], dtype=torch.long, device=tokens.device)
+        flat_positions = positions.reshape(-1).contiguous()
+        x, xn = E.embed_rmsnorm(tokens.reshape(-1).contiguous(), W["embed"], W["layers"][0]["attn_norm"], s.rms_eps)
+        for i in range(s.layers):
+            L = W["layers"][i]
+            after = W["layers"][i + 1]["attn_norm"] if i + 1 < s.layers else W["final_norm"]
+            q = E.qk_norm_rope_cache(kernels.dense(xn, wqkv[i]), L["q_norm"], L["k_norm"], s.rms_eps, s.clip_qkv, self.cos,
+                                     self.sin, flat_positions, slot, s.heads, s.kv_heads, s.head_dim, cache.k[i], cache.v[i])
+            a = F.scaled_dot_product_attention(q.view(B, T, s.heads, s.head_dim).transpose(1, 2),
+                                               cache.k[i, :, :, :start + T], cache.v[i, :, :, :start + T], attn_mask=mask,
+                                               enable_gqa=s.kv_heads != s.heads)
+            o = kernels.dense(a.transpose(1, 2).reshape(B * T, s.heads * s.head_dim), L["wo"])
+            x, h = E.add_rmsnorm(x, o, L["mlp_norm"], s.rms_eps, x_out=x)
+            if self._own_moe and s.top_k <= 64:
+                logits = F.linear(h, L["router"])
+                y, pos_of, idx = kernels.experts_rows(h, logits, L["gate_up"], L["down"], s.top_k, s.norm_topk_prob)
+                x, xn = E.combine_add_rmsnorm(y, pos_of, idx, x, after, s.rms_eps, x_out=x)
+            else:
+                x, xn = E.add_rmsnorm(x, self.moe(i, h).contiguous(), after, s.rms_eps, x_out=x)
+        cache.filled = start + T
+        cache.next_position = base + valid.long().sum(1)
+        return kernels.dense(xn.view(B, T, s.hidden)[:, -1].contiguous(), W["lm_head"])
+
+    def _prefill(self, tokens, cache, valid):
+        """Logits of the last prompt position [B, vocab], on the kernels where they apply."""
+        if self.fused:
+            return self.prefill_fused(tokens, cache, valid)
+        return self.forward(tokens, cache, valid)[:, -1]
 
     # ---- one decode step with every index on the device, so that it can be captured in a HIP graph
     @torch.no_grad()
@@ -316,7 +363,7 @@ class Decoder:
         if timings is not None:
             torch.cuda.synchronize()
             t0 = time.perf_counter()
-        first_logits = self.forward(tokens, cache, valid)[:, -1]
+        first_logits = self._prefill(tokens, cache, valid)
         if timings is not None:
             torch.cuda.synchronize()
             timings["prefill_s"] = time.perf_counter() - t0
@@ -382,7 +429,7 @@ class Decoder:
             valid[b, P - len(p):] = True
         tokens, valid = tokens.to(dev), valid.to(dev)
         cache = KVCache(self.s, B, P + max_new_tokens, dtype, dev)
-        logits = self.forward(tokens, cache, valid)[:, -1]
+        logits = self._prefill(tokens, cache, valid)
         first_logits = logits
         out = torch.zeros(B, max_new_tokens, dtype=torch.long, device=dev)
         steps = 0

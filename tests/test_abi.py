@@ -72,11 +72,13 @@ def test_decode_argument_errors_and_empty_batches(lib):
     assert lib.sy_combine_add_rmsnorm(None, None, None, 65, None, None, 1e-5, 4, 2048, None, None, None) == 1
     assert lib.sy_combine_add_rmsnorm(None, None, None, 8, None, None, 1e-5, 4, 2044, None, None, None) == 1
     assert lib.sy_combine_add_rmsnorm(None, None, None, 8, None, None, 1e-5, 0, 2048, None, None, None) == 0
-    assert lib.sy_qk_norm_rope_cache(None, None, None, 1e-5, 0.0, None, None, 64, None, None, 2, 16, 5, 128, 64, None, None,
-                                     None, None) == 1
-    assert lib.sy_qk_norm_rope_cache(None, None, None, 1e-5, 0.0, None, None, 64, None, None, 2, 16, 16, 72, 64, None, None,
-                                     None, None) == 1
-    assert lib.sy_qk_norm_rope_cache(None, None, None, 1e-5, 0.0, None, None, 64, None, None, 0, 16, 16, 128, 64, None,
+    assert lib.sy_qk_norm_rope_cache(None, None, None, 1e-5, 0.0, None, None, 64, None, None, 2, 1, 16, 5, 128, 64, None,
+                                     None, None, None) == 1
+    assert lib.sy_qk_norm_rope_cache(None, None, None, 1e-5, 0.0, None, None, 64, None, None, 2, 1, 16, 16, 72, 64, None,
+                                     None, None, None) == 1
+    assert lib.sy_qk_norm_rope_cache(None, None, None, 1e-5, 0.0, None, None, 64, None, None, 2, 0, 16, 16, 128, 64, None,
+                                     None, None, None) == 1
+    assert lib.sy_qk_norm_rope_cache(None, None, None, 1e-5, 0.0, None, None, 64, None, None, 0, 1, 16, 16, 128, 64, None,
                                      None, None, None) == 0
     assert lib.sy_decode_attention(None, None, None, None, None, 2, 16, 16, 96, 64, None, None) == 1
     assert b"64 or 128" in lib.sy_last_error()

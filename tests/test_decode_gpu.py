@@ -311,6 +311,42 @@ def test_a_step_on_the_decode_kernels_gives_the_logits_of_the_torch_step(batch, 
         assert int((per_seq > 2e-2).sum()) <= allowed and per_seq.max().item() < 0.3
 
 
+@pytest.mark.parametrize("batch,kw", [(6, {}), (5, {"kv_heads": 2, "clip_qkv": 0.5}), (3, {"head_dim": 128, "heads": 4, "kv_heads": 4}),
+                                      (40, {})])
+def test_prefill_on_the_kernels_gives_the_cache_and_last_logits_of_the_torch_prefill(batch, kw):
+    """A left-padded batch of prompts through `prefill_fused` and through `forward`: the same
+    mask, counters and positions; logits of the last position and the caches within the fp16
+    tolerance, up to the rare token whose router near-tie resolves the other way (its own keys
+    and values then differ; at most 1 % of the cached positions, and of the sequences' logits)."""
+    s, w, ps = model(7, batch, **kw)
+    fused = D.Decoder(s, w, max_positions=128, attention="kernels")
+    plain = D.Decoder(s, w, max_positions=128, attention="torch")
+    B, P = len(ps), max(len(p) for p in ps)
+    tokens = torch.zeros(B, P, dtype=torch.long)
+    valid = torch.zeros(B, P, dtype=torch.bool)
+    for b, p in enumerate(ps):
+        tokens[b, P - len(p):] = torch.tensor(p)
+        valid[b, P - len(p):] = True
+    tokens, valid = tokens.cuda(), valid.cuda()
+    ca, cb = (D.KVCache(s, B, P + 4, torch.float16, "cuda") for _ in range(2))
+    la = fused.prefill_fused(tokens, ca, valid)
+    lb = plain.forward(tokens, cb, valid)[:, -1]
+    assert la.shape == lb.shape == (B, s.vocab)
+    assert ca.filled == cb.filled == P and torch.equal(ca.next_position, cb.next_position) and torch.equal(ca.real, cb.real)
+    per_seq = (la.float() - lb.float()).abs().amax(-1)
+    assert int((per_seq > 2e-2).sum()) <= max(1, B // 100) and per_seq.max().item() < 0.3, per_seq
+    for a, b in ((ca.k, cb.k), (ca.v, cb.v)):
+        per_pos = ((a.float() - b.float()).abs() * cb.real[None, :, None, :, None]).amax((0, 2, 4))   # [B, capacity], real positions
+        assert (per_pos > 2e-2).float().mean().item() <= 0.01 and per_pos.max().item() < 0.5, per_pos.amax(1)
+    # appending a second chunk of tokens to the same caches works the same way
+    more = torch.randint(3, s.vocab, (B, 3), generator=torch.Generator().manual_seed(1)).cuda()
+    la2 = fused.prefill_fused(more, ca)
+    lb2 = plain.forward(more, cb)[:, -1]
+    per_seq = (la2.float() - lb2.float()).abs().amax(-1)
+    assert ca.filled == cb.filled == P + 3 and torch.equal(ca.next_position, cb.next_position)
+    assert int((per_seq > 2e-2).sum()) <= max(1, B // 100) and per_seq.max().item() < 0.3, per_seq
+
+
 def test_generation_on_the_decode_kernels_picks_the_torch_models_tokens_up_to_ties():
     """Greedy decoding through `step_fused`; every picked token is the PyTorch-attention
     model's top-1 for the same prefix, or within the logits tolerance of it."""
