@@ -9,8 +9,9 @@ Built for decode on one GPU: the KV cache is allocated once for the whole genera
 tables are precomputed, and the greedy loop keeps its tokens on the device, so a decode step
 is a queue of launches with no host read unless the caller asks for early stopping at `eos`.
 On a GPU in fp16 the attention side of a decode step runs on the library's decode kernels
-(`step_fused`: about ten launches per layer with the MoE layer's five, every projection a
-weight stream); prefill, fp32 and the CPU use the PyTorch operators (`forward`, `step_static`).
+(`step_fused`: eight launches per layer with the MoE layer's, every projection a weight
+stream) and a prompt goes through `prefill_fused` (the same row kernels around PyTorch's fused
+attention call); fp32 and the CPU use the PyTorch operators (`forward`, `step_static`).
 """
 
 from dataclasses import dataclass
