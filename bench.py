@@ -273,6 +273,13 @@ def run_sweep(args):
             return fn
 
         rec = {"tokens": N}
+        # the clocks of a GPU that sat idle while this size was set up need work to come back up
+        # (the first column measured would otherwise read several per cent slower than the others)
+        spin, spin_until = rotating("auto"), time.perf_counter() + SPIN_UP_MS / 1e3
+        while time.perf_counter() < spin_until:
+            for _ in range(10):
+                spin()
+            torch.cuda.synchronize()
         rec["auto_ms"] = med(rotating("auto"))
         rec["gemv_ms"] = med(rotating("gemv")) if N <= 1024 else None
         rec["gemm_ms"] = med(rotating("gemm"))
