@@ -3,21 +3,24 @@
 // a few dozen PyTorch launches per layer (switchyard/model.py:14-17 rmsnorm, :61-84
 // _attention, :117-121 attention_block); at decode each of them is a launch that moves a few
 // kilobytes, so the step is bound by launches, not by the 34 MB of attention weights and the
-// KV cache it has to read. Three kernels replace them (the projections themselves go through
+// KV cache it has to read. A few kernels replace them (the projections themselves go through
 // the weight-stream kernel with a single "expert"):
 //
-//   add_rmsnorm           x += delta; h = w * f16(x * rsqrt(mean(x^2) + eps)), one row per workgroup;
-//                         delta may be the combine of the MoE layer's rows (combine_add_rmsnorm),
-//                         and the router's logits of h may come out of the same launch
-//                         (add_rmsnorm_logits)
+//   row_kernel            one token per workgroup: x += delta; h = w * f16(x * rsqrt(mean(x^2) + eps)).
+//                         x may be an embedding lookup (embed_rmsnorm), delta may be the combine
+//                         of the MoE layer's rows (combine_add_rmsnorm), and the router's logits
+//                         of h may come out of the same launch (add_rmsnorm_logits)
 //   qk_norm_rope_cache    q/k RMS norm over the whole projection, clamp, rotary embedding, and
-//                         the new key and value written into the cache at `slot`
+//                         the new keys and values written into the cache from `slot` on (one
+//                         token per sequence at decode, the whole prompt at prefill)
 //   decode_attention      one query per (sequence, head) against the cache: a single pass over
 //                         the keys and values with a running softmax, HBM-bound; its _qkv form
 //                         does the work of qk_norm_rope_cache in its own prologue
+//   greedy_advance        arg-max of the logits, the token appended to the output, rotary
+//                         positions and cache slot advanced
 //
-// Everything a replayed HIP graph must not bake in (the cache slot, the rotary positions) is
-// read from device memory, so the same launches serve every step.
+// Everything a replayed HIP graph must not bake in (the cache slot, the rotary positions, the
+// output column) is read from device memory, so the same launches serve every step.
 //
 // Rounding follows the PyTorch graph on fp16 tensors where it is cheap to do so: the norm is
 // taken in fp32, rounded to fp16 and then scaled in fp16; rotary products and their sum are
