@@ -87,11 +87,16 @@ __device__ __forceinline__ bool find_tile(const int* __restrict__ offsets, int E
         const int lo = run + inc - mine;
         if (want >= lo && want < lo + mine) {
           const int height = ((last - first + mine - 1) / mine + 31) & ~31;
-          const int begin = first + (want - lo) * height;
+          // inside an expert the row tiles of one column tile follow each other: they stream the
+          // same weights, are equally high, and so start and finish together and meet in L2
+          const int within = (int)(logical - (long)lo * ncol_tiles);
+          const int col = BM == 256 ? within / mine : (int)(logical % ncol_tiles);
+          const int rt = BM == 256 ? within - col * mine : want - lo;
+          const int begin = first + rt * height;
           s_tile[0] = x;
           s_tile[1] = begin;
           s_tile[2] = min(begin + height, last);
-          s_tile[3] = (int)(logical % ncol_tiles);
+          s_tile[3] = col;
         }
         run += __shfl(inc, WAVE - 1, WAVE);
       }
