@@ -136,7 +136,8 @@ def torch_qk_step(qkv, L, s, cos, sin, positions, clip):
 
 
 @pytest.mark.parametrize("B,heads,kv_heads,hd,clip", [(8, 16, 16, 128, None), (3, 8, 2, 64, None), (64, 16, 16, 128, 0.4),
-                                                     (1, 4, 4, 64, None), (5, 32, 8, 128, 1.5)])
+                                                     (1, 4, 4, 64, None), (5, 32, 8, 128, 1.5),
+                                                     (2, 64, 64, 128, None)])        # the widest projection: 8192
 def test_qk_norm_rope_cache(B, heads, kv_heads, hd, clip):
     s = D.Shape(hidden=512, heads=heads, kv_heads=kv_heads, head_dim=hd, clip_qkv=clip)
     cap, max_pos, slot_at = 37, 96, 11
@@ -175,6 +176,8 @@ def test_qk_norm_rope_cache(B, heads, kv_heads, hd, clip):
     (2, 4, 4, 128, 9, 0),          # a single visible key
     (2, 4, 1, 64, 33, 2),
     (40, 16, 4, 64, 130, 129),
+    (2, 16, 16, 128, 4100, 4050),  # a long cache: 64 key groups per wavefront
+    (1, 1, 1, 64, 1, 0),           # one sequence, one head, a cache of one position
 ])
 def test_decode_attention(B, heads, kv_heads, hd, cap, slot_at):
     g = torch.Generator().manual_seed(11)
