@@ -39,8 +39,9 @@ T4_WEIGHT_GBS_AT_8 = 232.98490131032196  # the reference's published figure for 
 
 # HBM bytes per launch of the gate/up projection from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (scaled by a plain copy kernel of known size: 2.0 and 1.0), keyed by token count; the run is
-# summarised in profiles/decode_8tok_gemv_hbm_traffic.txt. Token counts not measured: None.
-MEASURED_TRAFFIC_BYTES = {8: 342.1e6}
+# summarised in profiles/decode_8tok_gemv_hbm_traffic.txt (8 tokens, the weight-stream kernel) and
+# profiles/prefill_4096tok_gemm.txt (4096 tokens, the 256-row MFMA tiles). Token counts not measured: None.
+MEASURED_TRAFFIC_BYTES = {8: 342.1e6, 4096: 869.7e6}
 SPIN_UP_MS = 50.0   # GPU kept busy this long before the warm-up steps (clock ramp of an idle GPU)
 
 
