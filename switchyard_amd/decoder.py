@@ -129,8 +129,9 @@ class KVCache:
 
 class Decoder:
     def __init__(self, shape, weights, moe=None, max_positions=4096, attention="auto"):
-        """attention: "kernels" (the decode kernels for one-token steps), "torch", or "auto":
-        kernels where they apply (GPU, fp16, head_dim 64 or 128)."""
+        """attention: "kernels" (the library's kernels for the decode step and around the prompt's
+        attention), "torch" (PyTorch operators throughout), or "auto": kernels where they apply
+        (GPU, fp16, head_dim 64 or 128)."""
         self.s, self.w = shape, weights
         self.moe = moe or self.kernel_moe
         self._own_moe = moe is None     # the step may then fold the layer's ends into its neighbours
