@@ -160,3 +160,15 @@ def test_graph_replayed_decode_equals_eager_decode():
     for _ in range(3):
         assert m.generate_graph(ps, 12) == eager
         assert m.generate(ps, 12) == eager
+
+
+def test_the_kernels_are_not_silently_replaced_on_the_cpu():
+    """attention="kernels" on weights the kernels cannot take (CPU, fp32) raises; "auto" there
+    means the PyTorch operators, and the default MoE hook has no CPU form at all."""
+    _, shape, weights = tiny("plain")
+    with pytest.raises(ValueError):
+        D.Decoder(shape, weights, max_positions=64, attention="kernels")
+    m = D.Decoder(shape, weights, max_positions=64)
+    assert m.fused is False
+    with pytest.raises(RuntimeError):
+        m.forward(torch.tensor([[3, 4, 5]]))      # the default hook calls the HIP kernels: CPU tensors are refused
