@@ -71,7 +71,16 @@ def load_library(path=LIB_PATH):
     return lib
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_device_index = getattr(torch._C, "_cuda_getDevice", None)
+
+
 def _stream():
+    """Raw handle of the current stream of the current device. torch.cuda.current_stream() builds
+    a Stream object on every call (2.8 us of host time per launch measured); the accessor torch
+    itself uses underneath returns the same handle in a fraction of that."""
+    if _raw_stream is not None and _device_index is not None:
+        return _raw_stream(_device_index())
     return torch.cuda.current_stream().cuda_stream
 
 
