@@ -34,6 +34,8 @@ SIGNATURES = {
     "sy_grouped_gemm": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int,
                                  _c_void_p, _c_void_p, _c_void_p]),
     "sy_combine": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p]),
+    "sy_moe_experts": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_int,
+                                _c_int] + [_c_void_p] * 11),
     "sy_add_rmsnorm": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_int, _c_int, _c_void_p, _c_void_p,
                                 _c_void_p]),
     "sy_embed_rmsnorm": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_float, _c_int, _c_int, _c_void_p, _c_void_p,
@@ -198,6 +200,32 @@ class Ext:
             raise RuntimeError("combine: pos_of / idx shorter than n_tokens * k")
         out = torch.empty((n_tokens, H), dtype=y.dtype, device=y.device)
         self._call(self.lib.sy_combine, y.data_ptr(), pos_of.data_ptr(), idx.data_ptr(), int(n_tokens), k, H,
+                   out.data_ptr(), _stream())
+        return out
+
+    def moe_experts(self, h, logits, gate_up, down, k, norm, mfma_tiles=False):
+        """route + sort, the two projections and combine in one call of the library (a decode
+        step: up to 256 tokens, 128 experts, top-8). h [N, H], logits [N, E] f16 -> out [N, H].
+        The intermediate results live in one scratch allocation and are not returned."""
+        _check(h, "h", torch.float16)
+        _check(logits, "logits", torch.float16)
+        _check(gate_up, "gate_up", torch.float16)
+        _check(down, "down", torch.float16)
+        N, H = h.shape
+        E, I = gate_up.shape[0], down.shape[2]
+        if tuple(logits.shape) != (N, E) or tuple(gate_up.shape) != (E, 2 * I, H) or tuple(down.shape) != (E, H, I):
+            raise RuntimeError("moe_experts: shapes of h / logits / gate_up / down do not match")
+        M = N * int(k)
+        sizes = [M * 4, M * 2, E * 4, (E + 1) * 4, M * 4, M * 2, M * 4, M * I * 2, M * H * 2]  # idx w counts offsets token wsorted pos_of act y
+        starts, at = [], 0
+        for size in sizes:
+            starts.append(at)
+            at += (size + 255) // 256 * 256
+        scratch = torch.empty(at, dtype=torch.uint8, device=h.device)
+        out = torch.empty((N, H), dtype=torch.float16, device=h.device)
+        base = scratch.data_ptr()
+        self._call(self.lib.sy_moe_experts, h.data_ptr(), logits.data_ptr(), N, E, int(k), int(bool(norm)),
+                   gate_up.data_ptr(), down.data_ptr(), H, I, int(bool(mfma_tiles)), *[base + s for s in starts],
                    out.data_ptr(), _stream())
         return out
 

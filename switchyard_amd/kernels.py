@@ -150,7 +150,13 @@ def experts_rows(h, logits, gate_up, down, top_k, norm_topk_prob, mode="auto"):
 def moe_layer(h, router, gate_up, down, top_k, norm_topk_prob, mode="auto"):
     N, n_experts = h.shape[0], gate_up.shape[0]
     if 0 < N <= FUSED_FRONT_MAX_TOKENS and n_experts <= 128 and top_k <= 8 and h.dtype == torch.float16:
-        y, pos_of, idx = experts_rows(h, F.linear(h, router).contiguous(), gate_up, down, top_k, norm_topk_prob, mode)
-        return ext().combine(y, pos_of, idx, N)
+        # one call of the library for everything after the router GEMM: the host pays for a call
+        # what the GPU needs for a small kernel, and the first projection would wait for it
+        if mode == "auto":
+            mode = _auto(N, N * top_k, n_experts)
+        if mode not in ("gemv", "gemm", "cublas"):
+            raise ValueError(f"unknown mode {mode!r}")
+        return ext().moe_experts(h.contiguous(), F.linear(h, router).contiguous(), gate_up, down, top_k, norm_topk_prob,
+                                 mfma_tiles=mode != "gemv")
     idx, w = route(h, router, top_k, norm_topk_prob)
     return experts(h, idx, w, gate_up, down, mode)

@@ -32,7 +32,7 @@ def test_header_declares_the_expected_entry_points():
     assert sorted(declared_symbols(HEADER)) == sorted(["sy_version", "sy_last_error", "sy_route", "sy_sort_workspace_bytes",
                                                   "sy_sort_by_expert", "sy_route_sort",
                                                   "sy_grouped_gemv", "sy_grouped_gemm",
-                                                  "sy_combine"])
+                                                  "sy_combine", "sy_moe_experts"])
 
 
 def test_library_exports_every_declared_symbol(lib):
@@ -45,9 +45,10 @@ def test_library_exports_every_declared_symbol(lib):
 
 def test_each_header_citation_names_a_reference_location():
     text = open(HEADER).read()
-    for name in ("sy_route", "sy_sort_by_expert", "sy_route_sort", "sy_grouped_gemv", "sy_grouped_gemm", "sy_combine"):
+    for name in ("sy_route", "sy_sort_by_expert", "sy_route_sort", "sy_grouped_gemv", "sy_grouped_gemm", "sy_combine",
+                 "sy_moe_experts"):
         comment = text[:text.index(f"SY_API int {name}(")].rsplit("/*", 1)[1]
-        assert re.search(r"moe_kernels\.cu:\d+", comment), name
+        assert re.search(r"(moe_kernels\.cu|kernels\.py):\d+", comment), name
 
 
 def test_each_decode_citation_names_a_reference_location():

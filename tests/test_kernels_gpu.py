@@ -406,3 +406,32 @@ def test_route_sort_limits(K):
         K.ext().route_sort(torch.zeros(300, 64, dtype=torch.float16, device=DEV), 8, False)   # too many tokens
     with pytest.raises(RuntimeError):
         K.ext().route_sort(torch.zeros(4, 64, dtype=torch.float16, device=DEV), 9, False)
+
+
+# ------------------------------------------------------------------ the experts of a decode step in one call
+@pytest.mark.parametrize("N,E,k,H,I", [(1, 64, 8, 2048, 1024), (8, 64, 8, 2048, 1024), (16, 64, 8, 2048, 1024),
+                                       (5, 16, 4, 128, 64), (40, 64, 8, 256, 128), (200, 64, 8, 256, 128)])
+@pytest.mark.parametrize("tiles", [False, True])
+@pytest.mark.parametrize("norm", [False, True])
+def test_experts_in_one_call_equal_the_five_calls(K, N, E, k, H, I, tiles, norm):
+    """sy_moe_experts enqueues what route_sort, the two projections and combine enqueue: the same
+    bits come out, with the weight-stream kernel and with the MFMA tiles; and a layer that
+    uses it agrees with the oracle's loop as the layer tests demand."""
+    h, router, gu, dn = cases.layer(N, E=E, k=k, H=H, I=I, seed=3, wstd=0.05)
+    h, router, gu, dn = (t.to(DEV) for t in (h, router, gu, dn))
+    logits = F.linear(h, router).contiguous()
+    ext = K.ext()
+    idx, w, counts, offsets, token, wsorted, pos_of = ext.route_sort(logits, k, norm)
+    M = N * k
+    if tiles:
+        act = ext.grouped_gemm(h, token, gu, offsets, None, 0, M, True, None)
+        y = ext.grouped_gemm(act, None, dn, offsets, None, 0, M, False, wsorted)
+    else:
+        act = ext.grouped_gemv(h, token, gu, offsets, M, True, None, N)
+        y = ext.grouped_gemv(act, None, dn, offsets, M, False, wsorted, N)
+    want = ext.combine(y, pos_of, idx, N)
+    got = ext.moe_experts(h, logits, gu, dn, k, norm, mfma_tiles=tiles)
+    assert torch.equal(got, want)
+    if N <= K.FUSED_FRONT_MAX_TOKENS:     # the layer takes this path: "gemv" and "gemm" name the kernels
+        layer = K.moe_layer(h, router, gu, dn, k, norm, mode="gemm" if tiles else "gemv")
+        assert torch.equal(layer, want)
