@@ -35,7 +35,7 @@ SIGNATURES = {
                                  _c_void_p, _c_void_p, _c_void_p]),
     "sy_combine": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p]),
     "sy_moe_experts": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_int,
-                                _c_int] + [_c_void_p] * 11),
+                                _c_int, _c_int] + [_c_void_p] * 11 + [_c_size_t, _c_void_p]),
     "sy_add_rmsnorm": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_int, _c_int, _c_void_p, _c_void_p,
                                 _c_void_p]),
     "sy_embed_rmsnorm": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_float, _c_int, _c_int, _c_void_p, _c_void_p,
@@ -203,10 +203,11 @@ class Ext:
                    out.data_ptr(), _stream())
         return out
 
-    def moe_experts(self, h, logits, gate_up, down, k, norm, mfma_tiles=False):
-        """route + sort, the two projections and combine in one call of the library (a decode
-        step: up to 256 tokens, 128 experts, top-8). h [N, H], logits [N, E] f16 -> out [N, H].
-        The intermediate results live in one scratch allocation and are not returned."""
+    def moe_experts(self, h, logits, gate_up, down, k, norm, mfma_tiles=False, one_launch_front=True):
+        """route and sort, the two projections and combine in one call of the library (at most
+        128 experts, top-8; one_launch_front needs at most 256 tokens). h [N, H], logits [N, E]
+        f16 -> out [N, H]. The intermediate results live in one scratch allocation and are not
+        returned."""
         _check(h, "h", torch.float16)
         _check(logits, "logits", torch.float16)
         _check(gate_up, "gate_up", torch.float16)
@@ -216,7 +217,9 @@ class Ext:
         if tuple(logits.shape) != (N, E) or tuple(gate_up.shape) != (E, 2 * I, H) or tuple(down.shape) != (E, H, I):
             raise RuntimeError("moe_experts: shapes of h / logits / gate_up / down do not match")
         M = N * int(k)
-        sizes = [M * 4, M * 2, E * 4, (E + 1) * 4, M * 4, M * 2, M * 4, M * I * 2, M * H * 2]  # idx w counts offsets token wsorted pos_of act y
+        need = 0 if one_launch_front else self.lib.sy_sort_workspace_bytes(N, int(k), E)
+        # idx w counts offsets token wsorted pos_of act y, then the sort's workspace
+        sizes = [M * 4, M * 2, E * 4, (E + 1) * 4, M * 4, M * 2, M * 4, M * I * 2, M * H * 2, need]
         starts, at = [], 0
         for size in sizes:
             starts.append(at)
@@ -225,8 +228,8 @@ class Ext:
         out = torch.empty((N, H), dtype=torch.float16, device=h.device)
         base = scratch.data_ptr()
         self._call(self.lib.sy_moe_experts, h.data_ptr(), logits.data_ptr(), N, E, int(k), int(bool(norm)),
-                   gate_up.data_ptr(), down.data_ptr(), H, I, int(bool(mfma_tiles)), *[base + s for s in starts],
-                   out.data_ptr(), _stream())
+                   gate_up.data_ptr(), down.data_ptr(), H, I, int(bool(mfma_tiles)), int(bool(one_launch_front)),
+                   *[base + s for s in starts[:9]], out.data_ptr(), base + starts[9] if need else None, need, _stream())
         return out
 
     # ---- the decode-step kernels around the MoE layer (include/switchyard_decode.h)

@@ -149,7 +149,7 @@ def experts_rows(h, logits, gate_up, down, top_k, norm_topk_prob, mode="auto"):
 
 def moe_layer(h, router, gate_up, down, top_k, norm_topk_prob, mode="auto"):
     N, n_experts = h.shape[0], gate_up.shape[0]
-    if 0 < N <= FUSED_FRONT_MAX_TOKENS and n_experts <= 128 and top_k <= 8 and h.dtype == torch.float16:
+    if N > 0 and n_experts <= 128 and top_k <= 8 and h.dtype == torch.float16:
         # one call of the library for everything after the router GEMM: the host pays for a call
         # what the GPU needs for a small kernel, and the first projection would wait for it
         if mode == "auto":
@@ -157,6 +157,6 @@ def moe_layer(h, router, gate_up, down, top_k, norm_topk_prob, mode="auto"):
         if mode not in ("gemv", "gemm", "cublas"):
             raise ValueError(f"unknown mode {mode!r}")
         return ext().moe_experts(h.contiguous(), F.linear(h, router).contiguous(), gate_up, down, top_k, norm_topk_prob,
-                                 mfma_tiles=mode != "gemv")
+                                 mfma_tiles=mode != "gemv", one_launch_front=N <= FUSED_FRONT_MAX_TOKENS)
     idx, w = route(h, router, top_k, norm_topk_prob)
     return experts(h, idx, w, gate_up, down, mode)

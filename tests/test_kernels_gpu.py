@@ -410,7 +410,8 @@ def test_route_sort_limits(K):
 
 # ------------------------------------------------------------------ the experts of a decode step in one call
 @pytest.mark.parametrize("N,E,k,H,I", [(1, 64, 8, 2048, 1024), (8, 64, 8, 2048, 1024), (16, 64, 8, 2048, 1024),
-                                       (5, 16, 4, 128, 64), (40, 64, 8, 256, 128), (200, 64, 8, 256, 128)])
+                                       (5, 16, 4, 128, 64), (40, 64, 8, 256, 128), (200, 64, 8, 256, 128),
+                                       (3000, 64, 8, 128, 64)])        # the sort with a workspace
 @pytest.mark.parametrize("tiles", [False, True])
 @pytest.mark.parametrize("norm", [False, True])
 def test_experts_in_one_call_equal_the_five_calls(K, N, E, k, H, I, tiles, norm):
@@ -421,7 +422,12 @@ def test_experts_in_one_call_equal_the_five_calls(K, N, E, k, H, I, tiles, norm)
     h, router, gu, dn = (t.to(DEV) for t in (h, router, gu, dn))
     logits = F.linear(h, router).contiguous()
     ext = K.ext()
-    idx, w, counts, offsets, token, wsorted, pos_of = ext.route_sort(logits, k, norm)
+    one_launch = N <= K.FUSED_FRONT_MAX_TOKENS
+    if one_launch:
+        idx, w, counts, offsets, token, wsorted, pos_of = ext.route_sort(logits, k, norm)
+    else:
+        idx, w = ext.route(logits, k, norm)
+        counts, offsets, token, wsorted, pos_of = ext.sort_by_expert(idx, w, E)
     M = N * k
     if tiles:
         act = ext.grouped_gemm(h, token, gu, offsets, None, 0, M, True, None)
@@ -430,8 +436,7 @@ def test_experts_in_one_call_equal_the_five_calls(K, N, E, k, H, I, tiles, norm)
         act = ext.grouped_gemv(h, token, gu, offsets, M, True, None, N)
         y = ext.grouped_gemv(act, None, dn, offsets, M, False, wsorted, N)
     want = ext.combine(y, pos_of, idx, N)
-    got = ext.moe_experts(h, logits, gu, dn, k, norm, mfma_tiles=tiles)
+    got = ext.moe_experts(h, logits, gu, dn, k, norm, mfma_tiles=tiles, one_launch_front=one_launch)
     assert torch.equal(got, want)
-    if N <= K.FUSED_FRONT_MAX_TOKENS:     # the layer takes this path: "gemv" and "gemm" name the kernels
-        layer = K.moe_layer(h, router, gu, dn, k, norm, mode="gemm" if tiles else "gemv")
-        assert torch.equal(layer, want)
+    layer = K.moe_layer(h, router, gu, dn, k, norm, mode="gemm" if tiles else "gemv")   # the layer takes this path
+    assert torch.equal(layer, want)
