@@ -43,6 +43,12 @@ SY_API int sy_embed_rmsnorm(const int64_t* tokens, const void* embed, int vocab,
 SY_API int sy_add_rmsnorm_logits(const void* x, const void* delta, const void* weight, float eps, const void* router,
                                  int E, int N, int H, void* x_out, void* h_out, void* logits, void* stream);
 
+/* The router GEMM alone, for a few rows (a decode step): replaces `F.linear(h, router)`
+ * (switchyard/kernels.py:30-32). h f16 [N,H]; router f16 [E,H] -> logits f16 [N,E], fp32 sums
+ * rounded once. One workgroup per row reads the whole router from L2, so this is for tens of
+ * rows, not thousands (the library GEMM takes over there). Limits: as sy_add_rmsnorm_logits. */
+SY_API int sy_router_logits(const void* h, const void* router, int N, int H, int E, void* logits, void* stream);
+
 /* sy_combine folded into the residual add and the next RMS norm: replaces combine()
  * (switchyard/csrc/moe_kernels.cu:435-444) followed by `x = x + moe(i, h)` and the rmsnorm of
  * the next block (switchyard/model.py:142,119 or :130).

@@ -96,19 +96,23 @@ SY_API int sy_grouped_gemm(const void* A, const int32_t* a_rows, const void* B, 
 SY_API int sy_combine(const void* y, const int32_t* pos_of, const int32_t* idx, int N, int k, int H, void* out,
                void* stream);
 
-/* Replaces experts() after the router GEMM (switchyard/kernels.py:76-88 with route():
- * sort -> pick -> ffn -> combine), in ONE call: route and sort (sy_route_sort when
- * one_launch_front is nonzero, else sy_route and sy_sort_by_expert with the given workspace), the
- * gate/up projection (SwiGLU, rows of h gathered through `token`), the down projection (x
- * router weight) and sy_combine are enqueued back to back, exactly as the separate calls would be.
- * h f16 [N,H]; logits f16 [N,E]; gate_up f16 [E,2I,H]; down f16 [E,H,I]; mfma_tiles 0 runs
- * sy_grouped_gemv twice, nonzero sy_grouped_gemm. Outputs as the separate calls' (idx, w, counts,
- * offsets, token, wsorted, pos_of), plus act f16 [N*k, I], y f16 [N*k, H] and out f16 [N,H],
- * all caller-allocated. Limits: those of the entry points it calls. */
-SY_API int sy_moe_experts(const void* h, const void* logits, int N, int E, int k, int norm, const void* gate_up,
-                          const void* down, int H, int I, int mfma_tiles, int one_launch_front, int32_t* idx, void* w,
-                          int32_t* counts, int32_t* offsets, int32_t* token, void* wsorted, int32_t* pos_of, void* act,
-                          void* y, void* out, void* sort_workspace, size_t sort_workspace_bytes, void* stream);
+/* Replaces moe_layer() (switchyard/kernels.py:91-93: route() with its router GEMM, :30-32, then
+ * experts(), :76-88: sort -> pick -> ffn -> combine) in ONE call: the router's logits
+ * (sy_router_logits, when `router` is given; with router NULL `logits` is an input), route and
+ * sort (sy_route_sort when one_launch_front is nonzero, else sy_route and sy_sort_by_expert with
+ * the given workspace), the gate/up projection (SwiGLU, rows of h gathered through `token`), the
+ * down projection (x router weight) and sy_combine are enqueued back to back, exactly as the
+ * separate calls would be.
+ * h f16 [N,H]; router f16 [E,H] or NULL; logits f16 [N,E]; gate_up f16 [E,2I,H]; down f16
+ * [E,H,I]; mfma_tiles 0 runs sy_grouped_gemv twice, nonzero sy_grouped_gemm. Outputs as the
+ * separate calls' (idx, w, counts, offsets, token, wsorted, pos_of), plus act f16 [N*k, I],
+ * y f16 [N*k, H] and out f16 [N,H], all caller-allocated. Limits: those of the entry points it
+ * calls. */
+SY_API int sy_moe_experts(const void* h, const void* router, void* logits, int N, int E, int k, int norm,
+                          const void* gate_up, const void* down, int H, int I, int mfma_tiles, int one_launch_front,
+                          int32_t* idx, void* w, int32_t* counts, int32_t* offsets, int32_t* token, void* wsorted,
+                          int32_t* pos_of, void* act, void* y, void* out, void* sort_workspace,
+                          size_t sort_workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

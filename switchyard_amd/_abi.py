@@ -34,8 +34,9 @@ SIGNATURES = {
     "sy_grouped_gemm": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int,
                                  _c_void_p, _c_void_p, _c_void_p]),
     "sy_combine": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p]),
-    "sy_moe_experts": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_int,
-                                _c_int, _c_int] + [_c_void_p] * 11 + [_c_size_t, _c_void_p]),
+    "sy_moe_experts": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p,
+                                _c_int, _c_int, _c_int, _c_int] + [_c_void_p] * 11 + [_c_size_t, _c_void_p]),
+    "sy_router_logits": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p]),
     "sy_add_rmsnorm": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_int, _c_int, _c_void_p, _c_void_p,
                                 _c_void_p]),
     "sy_embed_rmsnorm": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_float, _c_int, _c_int, _c_void_p, _c_void_p,
@@ -203,23 +204,34 @@ class Ext:
                    out.data_ptr(), _stream())
         return out
 
-    def moe_experts(self, h, logits, gate_up, down, k, norm, mfma_tiles=False, one_launch_front=True):
-        """route and sort, the two projections and combine in one call of the library (at most
-        128 experts, top-8; one_launch_front needs at most 256 tokens). h [N, H], logits [N, E]
-        f16 -> out [N, H]. The intermediate results live in one scratch allocation and are not
-        returned."""
+    def moe_experts(self, h, logits, gate_up, down, k, norm, mfma_tiles=False, one_launch_front=True, router=None):
+        """(The router's logits,) route and sort, the two projections and combine in one call of
+        the library (at most 128 experts, top-8; one_launch_front needs at most 256 tokens).
+        h [N, H] and either logits [N, E] f16 or router [E, H] f16 (then logits is None and the
+        library's own router kernel computes them: for tens of tokens) -> out [N, H]. The
+        intermediate results live in one scratch allocation and are not returned."""
         _check(h, "h", torch.float16)
-        _check(logits, "logits", torch.float16)
         _check(gate_up, "gate_up", torch.float16)
         _check(down, "down", torch.float16)
         N, H = h.shape
         E, I = gate_up.shape[0], down.shape[2]
-        if tuple(logits.shape) != (N, E) or tuple(gate_up.shape) != (E, 2 * I, H) or tuple(down.shape) != (E, H, I):
-            raise RuntimeError("moe_experts: shapes of h / logits / gate_up / down do not match")
+        if (logits is None) == (router is None):
+            raise RuntimeError("moe_experts: give the logits or the router")
+        if logits is not None:
+            _check(logits, "logits", torch.float16)
+            if tuple(logits.shape) != (N, E):
+                raise RuntimeError("moe_experts: logits must be [N, E]")
+        else:
+            _check(router, "router", torch.float16)
+            if tuple(router.shape) != (E, H):
+                raise RuntimeError("moe_experts: router must be [E, H]")
+        if tuple(gate_up.shape) != (E, 2 * I, H) or tuple(down.shape) != (E, H, I):
+            raise RuntimeError("moe_experts: shapes of h / gate_up / down do not match")
         M = N * int(k)
         need = 0 if one_launch_front else self.lib.sy_sort_workspace_bytes(N, int(k), E)
-        # idx w counts offsets token wsorted pos_of act y, then the sort's workspace
-        sizes = [M * 4, M * 2, E * 4, (E + 1) * 4, M * 4, M * 2, M * 4, M * I * 2, M * H * 2, need]
+        # idx w counts offsets token wsorted pos_of act y, then the sort's workspace and the logits
+        sizes = [M * 4, M * 2, E * 4, (E + 1) * 4, M * 4, M * 2, M * 4, M * I * 2, M * H * 2, need,
+                 N * E * 2 if logits is None else 0]
         starts, at = [], 0
         for size in sizes:
             starts.append(at)
@@ -227,10 +239,22 @@ class Ext:
         scratch = torch.empty(at, dtype=torch.uint8, device=h.device)
         out = torch.empty((N, H), dtype=torch.float16, device=h.device)
         base = scratch.data_ptr()
-        self._call(self.lib.sy_moe_experts, h.data_ptr(), logits.data_ptr(), N, E, int(k), int(bool(norm)),
+        self._call(self.lib.sy_moe_experts, h.data_ptr(), router.data_ptr() if router is not None else None,
+                   logits.data_ptr() if logits is not None else base + starts[10], N, E, int(k), int(bool(norm)),
                    gate_up.data_ptr(), down.data_ptr(), H, I, int(bool(mfma_tiles)), int(bool(one_launch_front)),
                    *[base + s for s in starts[:9]], out.data_ptr(), base + starts[9] if need else None, need, _stream())
         return out
+
+    def router_logits(self, h, router):
+        """h [N, H] @ router [E, H]^T -> logits [N, E] f16 by the library's own kernel (tens of rows)."""
+        _check(h, "h", torch.float16)
+        _check(router, "router", torch.float16)
+        if h.shape[1] != router.shape[1]:
+            raise RuntimeError("router_logits: h and router must have the same width")
+        logits = torch.empty((h.shape[0], router.shape[0]), dtype=torch.float16, device=h.device)
+        self._call(self.lib.sy_router_logits, h.data_ptr(), router.data_ptr(), h.shape[0], h.shape[1], router.shape[0],
+                   logits.data_ptr(), _stream())
+        return logits
 
     # ---- the decode-step kernels around the MoE layer (include/switchyard_decode.h)
     def add_rmsnorm(self, x, delta, weight, eps, x_out=None, router=None):

@@ -3,6 +3,7 @@
 #include <stdio.h>
 
 #include "common.h"
+#include "../../include/switchyard_decode.h"
 
 namespace {
 thread_local char g_error[512] = "";
@@ -39,20 +40,24 @@ extern "C" SY_API int sy_version(void) { return 200; }  // 0.2.0: the decode-ste
 
 extern "C" SY_API const char* sy_last_error(void) { return g_error; }
 
-// The experts of one layer in one call: route and sort, the two projections and combine,
-// enqueued back to back. Nothing here that the separate entry points do not do; it exists
+// The experts of one layer in one call: (the router's logits,) route and sort, the two
+// projections and combine, enqueued back to back. Nothing here that the separate entry points do not do; it exists
 // because a host binding pays several microseconds per call, and in front of the first
 // projection the GPU waits for exactly those (a layer of 8 tokens called once: 132 us with
 // five calls, the kernels themselves 102).
-extern "C" SY_API int sy_moe_experts(const void* h, const void* logits, int N, int E, int k, int norm, const void* gate_up,
+extern "C" SY_API int sy_moe_experts(const void* h, const void* router, void* logits, int N, int E, int k, int norm, const void* gate_up,
                                      const void* down, int H, int I, int mfma_tiles, int one_launch_front, int32_t* idx,
                                      void* w, int32_t* counts, int32_t* offsets, int32_t* token, void* wsorted,
                                      int32_t* pos_of, void* act, void* y, void* out, void* sort_workspace,
                                      size_t sort_workspace_bytes, void* stream) {
   SY_REQUIRE(N >= 0 && H >= 8 && I >= 8, "moe_experts: N = %d, H = %d, I = %d", N, H, I);
   if (N == 0) return SY_OK;
-  SY_REQUIRE(h && act && y && out, "moe_experts: null pointer");
+  SY_REQUIRE(h && logits && act && y && out, "moe_experts: null pointer");
   int rc;
+  if (router) {   // the router GEMM too: logits is then an output
+    rc = sy_router_logits(h, router, N, H, E, logits, stream);
+    if (rc) return rc;
+  }
   if (one_launch_front) {
     rc = sy_route_sort(logits, N, E, k, norm, idx, w, counts, offsets, token, wsorted, pos_of, stream);
   } else {

@@ -113,18 +113,27 @@ row_kernel(const half_t* x, const half_t* __restrict__ delta, const half_t* __re
       for (int j = 0; j < 8; ++j) ss += (float)v[i][j] * (float)v[i][j];
     }
   }
-  const float rs = rsqrtf(block_sum(ss, part, 0) / (float)H + eps);
+  if (LOGITS && !weight) {
+    // no norm asked for: the logits of the rows as they are (the router GEMM alone)
 #pragma unroll
-  for (int i = 0; i < MAX_CHUNKS; ++i) {
-    const int c = tid + i * nthreads;
-    if (c < chunks) {
-      const half8_t w = *reinterpret_cast<const half8_t*>(weight + c * 8);
-      half8_t h;
+    for (int i = 0; i < MAX_CHUNKS; ++i) {
+      const int c = tid + i * nthreads;
+      if (c < chunks) *reinterpret_cast<half8_t*>(hs + c * 8) = v[i];
+    }
+  } else {
+    const float rs = rsqrtf(block_sum(ss, part, 0) / (float)H + eps);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) h[j] = (half_t)((float)w[j] * (float)(half_t)((float)v[i][j] * rs));
-      if (x_out) *reinterpret_cast<half8_t*>(x_out + row + c * 8) = v[i];
-      *reinterpret_cast<half8_t*>(h_out + row + c * 8) = h;
-      if (LOGITS) *reinterpret_cast<half8_t*>(hs + c * 8) = h;
+    for (int i = 0; i < MAX_CHUNKS; ++i) {
+      const int c = tid + i * nthreads;
+      if (c < chunks) {
+        const half8_t w = *reinterpret_cast<const half8_t*>(weight + c * 8);
+        half8_t h;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) h[j] = (half_t)((float)w[j] * (float)(half_t)((float)v[i][j] * rs));
+        if (x_out) *reinterpret_cast<half8_t*>(x_out + row + c * 8) = v[i];
+        *reinterpret_cast<half8_t*>(h_out + row + c * 8) = h;
+        if (LOGITS) *reinterpret_cast<half8_t*>(hs + c * 8) = h;
+      }
     }
   }
   if (!LOGITS) return;
@@ -649,6 +658,17 @@ extern "C" SY_API int sy_add_rmsnorm_logits(const void* x, const void* delta, co
       (const half_t*)x, (const half_t*)delta, nullptr, nullptr, nullptr, 0, (const half_t*)weight, eps,
       (const half_t*)router, E, H, (half_t*)x_out, (half_t*)h_out, (half_t*)logits, nullptr, 0);
   return sy_check_launch("add_rmsnorm_logits");
+}
+
+extern "C" SY_API int sy_router_logits(const void* h, const void* router, int N, int H, int E, void* logits, void* stream) {
+  ROW_LIMITS("router_logits");
+  SY_REQUIRE(E >= 1 && E <= 1024, "router_logits: 1 <= E <= 1024 (got %d)", E);
+  if (N == 0) return SY_OK;
+  SY_REQUIRE(h && router && logits, "router_logits: null pointer");
+  row_kernel<false, true><<<N, 1024, (size_t)H * sizeof(half_t), (hipStream_t)stream>>>(
+      (const half_t*)h, nullptr, nullptr, nullptr, nullptr, 0, nullptr, 0.f, (const half_t*)router, E, H, nullptr, nullptr,
+      (half_t*)logits, nullptr, 0);
+  return sy_check_launch("router_logits");
 }
 
 extern "C" SY_API int sy_combine_add_rmsnorm(const void* y, const int32_t* pos_of, const int32_t* idx, int k, const void* x,

@@ -147,6 +147,14 @@ def experts_rows(h, logits, gate_up, down, top_k, norm_topk_prob, mode="auto"):
     return ffn(h, token, offsets, counts, wsorted, gate_up, down, idx.numel(), mode), pos_of, idx
 
 
+# Up to this many tokens the router's logits come from the library's own kernel, inside the same
+# call as everything else: it takes the GPU as long as the library GEMM (a layer of 8 tokens in
+# a stream of layers 102.0 us either way; the logits come out bit-equal), and the host does not
+# spend 18 us on a separate GEMM call (a layer called once: 116 us against 130). One workgroup
+# per token reads the whole router, so it is for tens of tokens.
+OWN_ROUTER_MAX_TOKENS = 64
+
+
 def moe_layer(h, router, gate_up, down, top_k, norm_topk_prob, mode="auto"):
     N, n_experts = h.shape[0], gate_up.shape[0]
     if N > 0 and n_experts <= 128 and top_k <= 8 and h.dtype == torch.float16:
@@ -156,7 +164,9 @@ def moe_layer(h, router, gate_up, down, top_k, norm_topk_prob, mode="auto"):
             mode = _auto(N, N * top_k, n_experts)
         if mode not in ("gemv", "gemm", "cublas"):
             raise ValueError(f"unknown mode {mode!r}")
-        return ext().moe_experts(h.contiguous(), F.linear(h, router).contiguous(), gate_up, down, top_k, norm_topk_prob,
-                                 mfma_tiles=mode != "gemv", one_launch_front=N <= FUSED_FRONT_MAX_TOKENS)
+        own = N <= OWN_ROUTER_MAX_TOKENS and h.shape[1] % 8 == 0 and h.shape[1] <= 8192
+        return ext().moe_experts(h.contiguous(), None if own else F.linear(h, router).contiguous(), gate_up, down, top_k,
+                                 norm_topk_prob, mfma_tiles=mode != "gemv", one_launch_front=N <= FUSED_FRONT_MAX_TOKENS,
+                                 router=router.contiguous() if own else None)
     idx, w = route(h, router, top_k, norm_topk_prob)
     return experts(h, idx, w, gate_up, down, mode)

@@ -420,8 +420,10 @@ def test_experts_in_one_call_equal_the_five_calls(K, N, E, k, H, I, tiles, norm)
     uses it agrees with the oracle's loop as the layer tests demand."""
     h, router, gu, dn = cases.layer(N, E=E, k=k, H=H, I=I, seed=3, wstd=0.05)
     h, router, gu, dn = (t.to(DEV) for t in (h, router, gu, dn))
-    logits = F.linear(h, router).contiguous()
     ext = K.ext()
+    # the logits the layer itself will route on: the library's own router kernel for tens of tokens
+    logits = ext.router_logits(h, router) if N <= K.OWN_ROUTER_MAX_TOKENS else F.linear(h, router).contiguous()
+    assert torch.allclose(logits.float(), h.float() @ router.float().T, rtol=2 ** -10, atol=1e-4)
     one_launch = N <= K.FUSED_FRONT_MAX_TOKENS
     if one_launch:
         idx, w, counts, offsets, token, wsorted, pos_of = ext.route_sort(logits, k, norm)
@@ -440,3 +442,6 @@ def test_experts_in_one_call_equal_the_five_calls(K, N, E, k, H, I, tiles, norm)
     assert torch.equal(got, want)
     layer = K.moe_layer(h, router, gu, dn, k, norm, mode="gemm" if tiles else "gemv")   # the layer takes this path
     assert torch.equal(layer, want)
+    if N <= K.OWN_ROUTER_MAX_TOKENS:     # and with the router GEMM inside the same call
+        assert torch.equal(ext.moe_experts(h, None, gu, dn, k, norm, mfma_tiles=tiles, one_launch_front=one_launch,
+                                           router=router), want)
