@@ -85,7 +85,8 @@ SY_API int sy_grouped_gemv(const void* A, const int32_t* a_rows, const void* B, 
  * MFMA tiles for many rows per expert. The row tiles of every expert are derived from
  * `offsets` inside the kernel, so the reference's tile_offsets / total_tiles arguments (and
  * the host read behind them, kernels.py:61) have no counterpart here.
- * Limits: K % 32 == 0. rows == 0 is a no-op. */
+ * Limits: K % 32 == 0; A under 2 GiB (its rows are addressed with 32-bit byte offsets; with
+ * a_rows the library cannot see A's size and the caller must keep to this). rows == 0 is a no-op. */
 SY_API int sy_grouped_gemm(const void* A, const int32_t* a_rows, const void* B, const int32_t* offsets, int E, int rows,
                     int Nout, int K, int swiglu, const void* scale, void* C, void* stream);
 

@@ -174,6 +174,8 @@ class Ext:
             raise RuntimeError("grouped: a_rows / scale shorter than rows")
         if a_rows is None and A.shape[0] < rows:
             raise RuntimeError("grouped: A has fewer rows than `rows`")
+        if a_rows is not None and A.numel() * 2 >= 2 ** 31:
+            raise RuntimeError("grouped: a gathered A must stay under 2 GiB (32-bit row offsets)")
         Nout = Nfull // 2 if swiglu else Nfull
         C = torch.empty((rows, Nout), dtype=A.dtype, device=A.device)
         extra = () if hint is None else (int(hint),)

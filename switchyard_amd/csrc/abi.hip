@@ -53,6 +53,8 @@ extern "C" SY_API int sy_moe_experts(const void* h, const void* router, void* lo
   SY_REQUIRE(N >= 0 && H >= 8 && I >= 8, "moe_experts: N = %d, H = %d, I = %d", N, H, I);
   if (N == 0) return SY_OK;
   SY_REQUIRE(h && logits && act && y && out, "moe_experts: null pointer");
+  // the projections address the gathered rows of h with 32-bit byte offsets
+  SY_REQUIRE((long)N * H * 2 < (1l << 31), "moe_experts: h must stay under 2 GiB (%d rows of %d)", N, H);
   int rc;
   if (router) {   // the router GEMM too: logits is then an output
     rc = sy_router_logits(h, router, N, H, E, logits, stream);

@@ -71,7 +71,8 @@ extern "C" SY_API int sy_route_sort(const void* logits, int N, int E, int k, int
   const size_t lds = sizeof(int) * (small_sort_lds_ints(E) + M) + sizeof(half_t) * M;
   hipStream_t st = (hipStream_t)stream;
   // one wavefront per token is all that the route needs when one wavefront sorts
-  const int threads = M <= WAVE ? N * WAVE : FRONT_THREADS;
+  // (the route loop strides by the wavefronts present, so fewer wavefronts than tokens is fine)
+  const int threads = M <= WAVE && N * WAVE <= FRONT_THREADS ? N * WAVE : FRONT_THREADS;
   if (E <= 64)
     front_kernel<1><<<1, threads, lds, st>>>((const half_t*)logits, N, E, k, norm, nbits, idx, (half_t*)w, counts,
                                                   offsets, token, (half_t*)wsorted, pos_of);

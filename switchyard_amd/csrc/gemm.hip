@@ -331,7 +331,7 @@ __device__ __forceinline__ void load_to_lds(int4_t rsrc, unsigned voffset, unsig
       "buffer_load_dwordx4 %1, %2, %3 offen lds"
       :
       : "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset)
-      : "memory");  // m0 is not otherwise used in this file: the compiler needs it for no LDS or lane instruction here
+      : "memory", "m0");
 }
 
 // WN wavefronts side by side over the weight rows, two over the rows: 2 x 4 wavefronts of 128 rows x

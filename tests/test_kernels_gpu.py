@@ -379,7 +379,8 @@ def test_full_size_properties(K, olmoe, N, mode):
 
 # ------------------------------------------------------------------ route + sort in one launch (decode)
 @pytest.mark.parametrize("N,E,k,H", [(1, 64, 8, 2048), (8, 64, 8, 2048), (33, 64, 8, 2048), (64, 64, 8, 256),
-                                     (256, 64, 8, 256), (7, 128, 8, 512), (20, 16, 4, 128), (5, 60, 3, 64)])
+                                     (256, 64, 8, 256), (7, 128, 8, 512), (20, 16, 4, 128), (5, 60, 3, 64),
+                                     (20, 16, 3, 128), (64, 64, 1, 256)])   # more tokens than wavefronts, one-wavefront sort
 @pytest.mark.parametrize("norm", [False, True])
 def test_route_sort_in_one_launch(K, N, E, k, H, norm):
     """Bit for bit what route followed by sort_by_expert gives, and what the oracle gives."""
