@@ -11,7 +11,8 @@
  *   - "f16" is IEEE binary16; every matrix is row-major and contiguous;
  *   - the return value is 0 on success, otherwise an SY_ERR_* code, and sy_last_error()
  *     returns a message for the calling thread;
- *   - calls are re-entrant; the library keeps no state between calls.
+ *   - calls are re-entrant and the library keeps no state between calls (the one exception,
+ *     sy_sort_by_expert_static, says so).
  */
 #ifndef SWITCHYARD_MOE_H
 #define SWITCHYARD_MOE_H
@@ -58,6 +59,21 @@ SY_API size_t sy_sort_workspace_bytes(int N, int k, int E);
 SY_API int sy_sort_by_expert(const int32_t* idx, const void* w, int w_bytes, int N, int k, int E, int32_t* counts,
                       int32_t* offsets, int32_t* token, void* wsorted, int32_t* pos_of, void* workspace,
                       size_t workspace_bytes, void* stream);
+
+/* sy_sort_by_expert for callers that cannot allocate (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc). It has no counterpart in the reference, whose
+ * sort allocates with ATen inside the call (moe_kernels.cu:146-152). Same arguments and results
+ * as sy_sort_by_expert without the workspace: the per-wavefront histograms live in a static
+ * device array of SY_SORT_STATIC_BYTES inside the library (one copy per GPU, held until the
+ * process ends). Calls whose sy_sort_workspace_bytes() exceeds that return SY_ERR_ARG (with 64
+ * experts the array covers about two million choices). Every call on a GPU uses that GPU's one
+ * array: calls that overlap on one GPU (two streams, two threads) race; calls on one stream do
+ * not. The array's address is looked up on the first call on each device; make that call
+ * outside a graph capture. */
+#define SY_SORT_STATIC_BYTES (1 << 20)
+SY_API int sy_sort_by_expert_static(const int32_t* idx, const void* w, int w_bytes, int N, int k, int E,
+                                    int32_t* counts, int32_t* offsets, int32_t* token, void* wsorted,
+                                    int32_t* pos_of, void* stream);
 
 /* Route and sort of a decode step in ONE launch (one workgroup).
  * Fuses route() (moe_kernels.cu:73-89) and sort_by_expert() (moe_kernels.cu:142-157), which the

@@ -27,6 +27,8 @@ SIGNATURES = {
     "sy_sort_workspace_bytes": (_c_size_t, [_c_int, _c_int, _c_int]),
     "sy_sort_by_expert": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p,
                                    _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_size_t, _c_void_p]),
+    "sy_sort_by_expert_static": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p,
+                                          _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
     "sy_route_sort": (_c_int, [_c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                                _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
     "sy_grouped_gemv": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int,

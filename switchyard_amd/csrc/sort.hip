@@ -20,11 +20,40 @@
 //
 // Replaces count_kernel / assign_kernel / sort_by_expert of the reference
 // (switchyard/csrc/moe_kernels.cu:91-157).
+#include <mutex>
+
 #include "sort_core.h"
 
 namespace {
 
 using namespace sort_core;
+
+// Workspace of sy_sort_by_expert_static: the per-wavefront histograms of the launches over many
+// workgroups, for callers that cannot allocate. Every GPU the library runs on holds its own
+// copy of this array until the process ends. In host code the array's name is only a handle
+// for hipGetSymbolAddress, never a device address: launches take static_scratch()'s pointer.
+static __device__ __align__(256) unsigned char scratch[SY_SORT_STATIC_BYTES];
+
+constexpr int MAX_DEVICES = 64;
+std::mutex scratch_mutex;
+void* scratch_ptr[MAX_DEVICES] = {nullptr};
+
+// Address of `scratch` on the current device, resolved once per device.
+int static_scratch(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES)
+    return sy_fail(SY_ERR_LAUNCH, "sort_by_expert_static: no current device below %d", MAX_DEVICES);
+  std::lock_guard<std::mutex> hold(scratch_mutex);
+  if (!scratch_ptr[dev]) {
+    void* p = nullptr;
+    const hipError_t err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || !p)
+      return sy_fail(SY_ERR_LAUNCH, "sort_by_expert_static: hipGetSymbolAddress: %s", hipGetErrorString(err));
+    scratch_ptr[dev] = p;
+  }
+  *out = scratch_ptr[dev];
+  return SY_OK;
+}
 
 // ---------------------------------------------------------------- one workgroup does it all
 template <typename W>
@@ -177,4 +206,22 @@ extern "C" SY_API int sy_sort_by_expert(const int32_t* idx, const void* w, int w
                                  (hipStream_t)stream);
   return launch_sort<uint32_t>(idx, w, M, k, E, counts, offsets, token, wsorted, pos_of, workspace,
                                (hipStream_t)stream);
+}
+
+// The same sort with the histograms in the library's own static device array instead of a
+// workspace argument. The first launch overwrites every word of the array that the second one
+// reads, so nothing has to be cleared between calls.
+extern "C" SY_API int sy_sort_by_expert_static(const int32_t* idx, const void* w, int w_bytes, int N, int k, int E,
+                                               int32_t* counts, int32_t* offsets, int32_t* token, void* wsorted,
+                                               int32_t* pos_of, void* stream) {
+  SY_REQUIRE(N >= 0 && k >= 1 && E >= 1, "sort_by_expert_static: N = %d, k = %d, E = %d", N, k, E);
+  const size_t need = sy_sort_workspace_bytes(N, k, E);
+  SY_REQUIRE(need <= (size_t)SY_SORT_STATIC_BYTES,
+             "sort_by_expert_static: N*k = %ld choices over %d experts need %zu bytes of histograms, the static "
+             "array holds %d; use sy_sort_by_expert with a workspace",
+             (long)N * k, E, need, SY_SORT_STATIC_BYTES);
+  void* ws = nullptr;
+  if (need)
+    if (int rc = static_scratch(&ws)) return rc;
+  return sy_sort_by_expert(idx, w, w_bytes, N, k, E, counts, offsets, token, wsorted, pos_of, ws, need, stream);
 }

@@ -30,7 +30,7 @@ def test_header_declares_the_expected_entry_points():
                                                        "sy_greedy_advance", "sy_qk_norm_rope_cache", "sy_router_logits"]
     assert sorted(os.listdir(os.path.join(ROOT, "include"))) == ["switchyard_decode.h", "switchyard_moe.h"]
     assert sorted(declared_symbols(HEADER)) == sorted(["sy_version", "sy_last_error", "sy_route", "sy_sort_workspace_bytes",
-                                                  "sy_sort_by_expert", "sy_route_sort",
+                                                  "sy_sort_by_expert", "sy_sort_by_expert_static", "sy_route_sort",
                                                   "sy_grouped_gemv", "sy_grouped_gemm",
                                                   "sy_combine", "sy_moe_experts"])
 
@@ -45,7 +45,7 @@ def test_library_exports_every_declared_symbol(lib):
 
 def test_each_header_citation_names_a_reference_location():
     text = open(HEADER).read()
-    for name in ("sy_route", "sy_sort_by_expert", "sy_route_sort", "sy_grouped_gemv", "sy_grouped_gemm", "sy_combine",
+    for name in ("sy_route", "sy_sort_by_expert", "sy_sort_by_expert_static", "sy_route_sort", "sy_grouped_gemv", "sy_grouped_gemm", "sy_combine",
                  "sy_moe_experts"):
         comment = text[:text.index(f"SY_API int {name}(")].rsplit("/*", 1)[1]
         assert re.search(r"(moe_kernels\.cu|kernels\.py):\d+", comment), name
@@ -100,6 +100,11 @@ def test_argument_errors_are_reported_without_a_device(lib):
     assert lib.sy_combine(None, None, None, 4, 65, 2048, None, None) == 1
     assert lib.sy_sort_by_expert(None, None, 3, 4, 8, 64, None, None, None, None, None, None, 0, None) == 1
     assert lib.sy_sort_by_expert(None, None, 2, 4, 8, 513, None, None, None, None, None, None, 0, None) == 1
+    # the static array holds 1 MiB of histograms: 160 000 choices over 512 experts need more
+    assert lib.sy_sort_workspace_bytes(20000, 8, 512) > (1 << 20)
+    assert lib.sy_sort_by_expert_static(None, None, 2, 20000, 8, 512, None, None, None, None, None, None) == 1
+    assert b"static" in lib.sy_last_error()
+    assert lib.sy_sort_by_expert_static(None, None, 3, 4, 8, 64, None, None, None, None, None, None) == 1
 
 
 def test_empty_inputs_are_no_ops(lib):
