@@ -10,12 +10,16 @@ tokens, the configuration the reference's headline is quoted on. The metric is t
 counted once, over the layer time. Successive steps rotate through several layers' weights, as
 a decoder does, so that no step finds its weights in the 256 MB last-level cache.
 
-Prints ONE JSON line with the metric, a `roofline` object for the dominant kernel (the
-gate/up projection: two thirds of the weight bytes), timed per launch with events on the
-launch stream, a `cpu_baseline` object: the per-expert PyTorch loop on this host's cores, and (in
-the default configuration) a `decode` object: tokens/s of the full 16-layer model's greedy decode
-at batch 8 and 64, the second half of the reference's headline (`--decode 8,64` gives the detailed
-lines with the comparison against the per-expert loop in the hook)."""
+Prints ONE JSON line. Besides the contract's fields (decode at 8 tokens, timed as a stream of
+layer calls) it carries: the same figure by the reference's timing method (`*_event_median`); a
+`roofline` object for the dominant kernel (the gate/up projection: two thirds of the weight
+bytes) and one for the down projection, each timed per launch with events on the launch stream;
+a `cpu_baseline` object: the per-expert PyTorch loop on this host's cores; `gpu_loop_fp16`: the
+same loop on the GPU; and, in the default configuration, `decode_sizes` (1, 8, 16, 32 tokens),
+`prefill` (4096 tokens on the MFMA tiles with its own `roofline`, bound "mfma"; 256 and 1024
+tokens beside it) and `decode`: tokens/s of the full 16-layer model's greedy decode at batch 8 and
+64 with the step's byte roofline, the MoE share and the top-1 check against the per-expert loop
+(`--decode 8,64` prints more detail per batch)."""
 
 import argparse
 import json
@@ -36,13 +40,34 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published
 EXPERT_BYTES = 3 * H * I * 2   # gate + up + down of one expert, fp16
 T4_WEIGHT_GBS_AT_8 = 232.98490131032196  # the reference's published figure for this metric (Tesla T4)
-
-# HBM bytes per launch of the gate/up projection from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (scaled by a plain copy kernel of known size: 2.0 and 1.0), keyed by token count; the run is
-# summarised in profiles/decode_8tok_gemv_hbm_traffic.txt (8 tokens, the weight-stream kernel) and
-# profiles/prefill_4096tok_gemm.txt (4096 tokens, the 256-row MFMA tiles). Token counts not measured: None.
-MEASURED_TRAFFIC_BYTES = {8: 342.1e6, 4096: 869.7e6}
 SPIN_UP_MS = 50.0   # GPU kept busy this long before the warm-up steps (clock ramp of an idle GPU)
+DECODE_SIZES = (1, 8, 16, 32)        # the decode configuration's token counts
+PREFILL_SIZES = (256, 1024, 4096)    # the prefill configuration's token counts
+TIMING = ("value, us_per_layer: K layer calls issued back to back between two synchronizes (a stream of layers, as a "
+          "decoder issues them); *_event_median: one event pair around each single call, median of 20 after 3 "
+          "warm-ups (the reference's bench/kernels.py:13-26), which adds the launch latency of an idle queue")
+
+
+def measured_traffic(tokens, kernel):
+    """HBM bytes per launch from a committed rocprofv3 FETCH_SIZE / WRITE_SIZE summary, or None.
+    A summary under profiles/ ends with lines `bench-traffic: tokens=N kernel=NAME bytes=B file=SHA16`
+    naming the kernel source it was taken from and the first 16 hex digits of its SHA-256; a figure
+    whose source has changed since (or a missing summary) is not reported."""
+    import glob
+    import hashlib
+
+    for path in glob.glob(os.path.join(ROOT, "profiles", "*.txt")):
+        for line in open(path):
+            if not line.startswith("bench-traffic:"):
+                continue
+            f = dict(x.split("=", 1) for x in line.split()[1:])
+            if int(f["tokens"]) != tokens or f["kernel"] != kernel:
+                continue
+            name, sha = f["file"].split(":")
+            src = os.path.join(ROOT, "switchyard_amd", "csrc", name)
+            if os.path.exists(src) and hashlib.sha256(open(src, "rb").read()).hexdigest()[:16] == sha:
+                return float(f["bytes"])
+    return None
 
 
 def make_layers(n_layers, seed=0):
@@ -89,6 +114,149 @@ def stream_times(fn, reps, group=10):
     return [ev[i].elapsed_time(ev[i + 1]) / group for i in range(n)]
 
 
+def spin_up(fn, ms=SPIN_UP_MS):
+    """The clocks of an idle GPU take some milliseconds of work to come up (20 launches after an
+    idle gap run several per cent slower than the same launches in a long stream), so the GPU is
+    kept busy with the calls about to be timed; nothing of it is timed."""
+    until = time.perf_counter() + ms / 1e3
+    while time.perf_counter() < until:
+        for _ in range(10):
+            fn()
+        torch.cuda.synchronize()
+
+
+def routed_ids(kernels, h, router):
+    """Expert ids exactly as kernels.moe_layer routes them: up to OWN_ROUTER_MAX_TOKENS tokens the
+    logits come from the library's own router kernel, above that from F.linear."""
+    if h.shape[0] <= kernels.OWN_ROUTER_MAX_TOKENS:
+        logits = kernels.ext().router_logits(h, router)
+    else:
+        logits = F.linear(h, router).contiguous()
+    return kernels.ext().route(logits, TOPK, False)
+
+
+def experts_used(kernels, h, layers):
+    """Experts that receive a token, per layer (the numerator of the reference's metric)."""
+    out = []
+    for router, _, _ in layers:
+        idx, _ = routed_ids(kernels, h, router)
+        out.append(int((torch.bincount(idx.flatten().long(), minlength=E) > 0).sum()))
+    return out
+
+
+def time_layer(kernels, h, layers, mode, steps, warmup, spin=True):
+    """One kernels.moe_layer call per step, rotating through `layers`: (ms per step of a stream
+    of steps, median ms of event-timed single calls, used experts per layer)."""
+    calls = [0]
+
+    def step():
+        router, gu, dn = layers[calls[0] % len(layers)]
+        calls[0] += 1
+        return kernels.moe_layer(h, router, gu, dn, TOPK, False, mode)
+
+    if spin:
+        spin_up(step)
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    calls[0] = 0
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms_stream = (time.perf_counter() - t0) * 1e3 / steps
+    calls[0] = 0
+    for _ in range(3):
+        step()
+    torch.cuda.synchronize()
+    calls[0] = 0   # every event-timed call is layer 0, so its used-expert count is known exactly
+    single = lambda: kernels.moe_layer(h, *layers[0], TOPK, False, mode)
+    ms_event = statistics.median(event_times(single, 20))
+    return ms_stream, ms_event
+
+
+def layer_record(kernels, N, layers, mode, steps, warmup):
+    """Layer time and both roofline fractions at N tokens."""
+    h = hidden(N).to("cuda:0")
+    used = experts_used(kernels, h, layers)
+    ms_stream, ms_event = time_layer(kernels, h, layers, mode, steps, warmup)
+    used_mean = sum(used[j % len(layers)] for j in range(steps)) / steps
+    flops = N * TOPK * 6 * H * I
+    gbs, gbs_ev = used_mean * EXPERT_BYTES / ms_stream / 1e6, used[0] * EXPERT_BYTES / ms_event / 1e6
+    tf = flops / ms_stream / 1e9
+    return {"tokens": N, "mode": mode if mode != "auto" else kernels._auto(N, N * TOPK, E), "us_per_layer": ms_stream * 1e3,
+            "us_per_layer_event_median": ms_event * 1e3, "experts_used_mean": used_mean, "experts_used_layer0": used[0],
+            "weight_GBps": gbs, "weight_GBps_event_median": gbs_ev, "frac_of_hbm_peak": gbs / HBM_PEAK_GBS,
+            "frac_of_hbm_peak_event_median": gbs_ev / HBM_PEAK_GBS, "tflops": tf,
+            "frac_of_mfma_peak": tf / MFMA_F16_PEAK_TFLOPS,
+            "binding_roofline": "mfma" if flops / (MFMA_F16_PEAK_TFLOPS * 1e12) > used_mean * EXPERT_BYTES / (HBM_PEAK_GBS * 1e9) else "hbm"}
+
+
+def projection_times(kernels, N, layers, mode, reps, warmup):
+    """The two grouped projections of the layer, each timed per launch in a stream of launches
+    of that kernel alone (events on the launch stream), rotating through the layers' weights.
+    Returns (gate/up ms, down ms, used experts per layer, whether the weight-stream kernel ran)."""
+    dev = "cuda:0"
+    h = hidden(N).to(dev)
+    M = N * TOPK
+    use_gemv = (mode if mode != "auto" else kernels._auto(N, M, E)) == "gemv"
+    rot, used = [], []
+    for router, gu, dn in layers:
+        idx, w = routed_ids(kernels, h, router)
+        counts, offsets, token, wsorted, pos_of = kernels.ext().sort_by_expert(idx, w, E)
+        used.append(int((counts > 0).sum()))
+        rot.append((gu, dn, offsets, token, wsorted))
+    act = torch.randn(M, I, generator=torch.Generator().manual_seed(7)).mul_(0.3).half().to(dev)
+    calls = [0]
+    X = kernels.ext()
+
+    def gate_up():
+        gu, _, off, tok, _ = rot[calls[0] % len(rot)]
+        calls[0] += 1
+        return X.grouped_gemv(h, tok, gu, off, M, True, None, N) if use_gemv else X.grouped_gemm(h, tok, gu, off, None, 0, M, True, None)
+
+    def down():
+        _, dn, off, _, ws = rot[calls[0] % len(rot)]
+        calls[0] += 1
+        return X.grouped_gemv(act, None, dn, off, M, False, ws, N) if use_gemv else X.grouped_gemm(act, None, dn, off, None, 0, M, False, ws)
+
+    out = []
+    for fn in (gate_up, down):
+        spin_up(fn, 20.0)
+        for _ in range(max(3, warmup)):
+            fn()
+        calls[0] = 0
+        t = stream_times(fn, max(reps, 20), 10)
+        out.append(sum(t) / len(t))
+    return out[0], out[1], used, use_gemv
+
+
+def projection_rooflines(kernels, N, layers, mode, reps, warmup):
+    """`roofline` objects of the gate/up projection (the dominant kernel) and of the down
+    projection at N tokens. Bound and algorithmic figure: below about 300 rows per expert the
+    launch is a stream over the used experts' weights (bytes, against HBM peak), above it is
+    bound by the MFMAs (flops, against dense fp16 peak)."""
+    gu_ms, dn_ms, used, use_gemv = projection_times(kernels, N, layers, mode, reps, warmup)
+    used_mean = sum(used) / len(used)
+    M = N * TOPK
+    out = []
+    for name, ms, share, src in (("gate/up", gu_ms, 2, "gate_up"), ("down", dn_ms, 1, "down")):
+        if use_gemv or M // E < 300:
+            alg = used_mean * share * H * I * 2
+            roof = {"bound": "hbm", "achieved": alg / ms / 1e6, "peak": HBM_PEAK_GBS, "unit": "GB/s"}
+        else:
+            alg = M * share * 2 * H * I
+            roof = {"bound": "mfma", "achieved": alg / ms / 1e9, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s"}
+        roof["frac"] = roof["achieved"] / roof["peak"]
+        roof["traffic"] = measured_traffic(N, ("gemv_" if use_gemv else "gemm_") + src)
+        epi = "swiglu" if share == 2 else "scale"
+        roof["kernel"] = f"{'gemv_kernel' if use_gemv else 'grouped_gemm'}<{epi}> ({name} projection)"
+        roof["us_per_launch"] = ms * 1e3
+        roof["algorithmic_per_launch"] = alg
+        out.append(roof)
+    return out[0], out[1]
+
+
 def cpu_loop_baseline(h, router, gu, dn, used, reps=5):
     """The reference per-expert loop (switchyard/moe.py:34-42) restated in oracle/, fp32, on the host."""
     from oracle import moe_oracle as O
@@ -108,25 +276,102 @@ def cpu_loop_baseline(h, router, gu, dn, used, reps=5):
             "us_per_layer": t * 1e6}
 
 
+def gpu_loop_baseline(layers, sizes=(8, 4096)):
+    """The reference's "loop" column (bench/kernels.py:41): the same per-expert PyTorch loop in fp16
+    on the GPU, event-timed like the kernels (median of 5 after 1 warm-up), ms per layer."""
+    from oracle import moe_oracle as O
+
+    router, gu, dn = layers[0]
+    out = {}
+    for N in sizes:
+        h = hidden(N).to("cuda:0")
+        idx, w = O.route(h, router, TOPK, False)
+        O.experts_loop(h, idx, w, gu, dn)
+        torch.cuda.synchronize()
+        out[str(N)] = {"ms_per_layer": statistics.median(event_times(lambda: O.experts_loop(h, idx, w, gu, dn), 5))}
+    return out
+
+
 def decode_rates(batches=(8, 64), prompt_len=512, new_tokens=128):
     """The other half of the headline metric: greedy decode of the full OLMoE-1B-7B-shaped model
-    (16 layers, random fp16 weights), HIP-graph replay of the step, tokens/s per batch size."""
+    (16 layers, random fp16 weights). Per batch size: tokens/s with the decode step on the
+    library's kernels (HIP-graph replay of Decoder.step_fused), tokens/s of the configuration as
+    written (attention in PyTorch operators, the MoE layers through the hook ->
+    kernels.moe_layer; the step replayed as a graph as well), the bytes a step must read and the
+    fraction of HBM peak that makes of the step time, the MoE layers' share of the step, and
+    whether the first generated token is the top-1 of the same model with the per-expert
+    PyTorch loop in the hook, for every row."""
+    from oracle import moe_oracle as O
     from switchyard_amd import decoder as D
+    from switchyard_amd import kernels
 
+    dev = torch.device("cuda:0")
     s = D.OLMOE_1B_7B
-    w = D.random_weights(s, device="cuda:0", seed=0)
-    model = D.Decoder(s, w, max_positions=prompt_len + new_tokens + 8)
+    w = D.random_weights(s, device=dev, seed=0)
+    cap = prompt_len + new_tokens + 8
+    model = D.Decoder(s, w, max_positions=cap)
+    as_written = D.Decoder(s, w, max_positions=cap, attention="torch")      # self.moe = the hook -> kernels.moe_layer
+
+    def loop_moe(i, h):
+        L = w["layers"][i]
+        return O.moe_layer(h, L["router"], L["gate_up"], L["down"], s.top_k, s.norm_topk_prob)
+
+    loop_model = D.Decoder(s, w, moe=loop_moe, max_positions=cap, attention="torch")
+    layers = [(L["router"], L["gate_up"], L["down"]) for L in w["layers"]]
+    attn_bytes = s.layers * (2 * s.heads + 2 * s.kv_heads) * s.head_dim * s.hidden * 2
+    head_bytes = s.vocab * s.hidden * 2
+    router_bytes = s.layers * s.experts * s.hidden * 2
     out = {"model": "OLMoE-1B-7B shape, 16 layers, random-init fp16", "prompt_len": prompt_len,
-           "new_tokens": new_tokens, "step": "HIP-graph replay of Decoder.step_fused"}
+           "new_tokens": new_tokens, "step": "HIP-graph replay of Decoder.step_fused (every launch a kernel of this library)",
+           "as_written_step": "HIP-graph replay of Decoder.step_static: attention in PyTorch operators, MoE through the hook",
+           "bytes_per_step": "used experts' weights of 16 layers + attention, router and lm_head weights + the KV cache "
+                             "at the mean length of the run; roofline_frac = bytes / 8 TB/s / step time"}
     for B in batches:
         prompts = torch.randint(3, s.vocab, (B, prompt_len), generator=torch.Generator().manual_seed(0)).tolist()
+        tokens = torch.tensor(prompts, device=dev)
         model.generate(prompts, 4)
         torch.cuda.synchronize()
         tm = {}
-        model.generate_graph(prompts, new_tokens + 1, timings=tm)
-        out[f"b{B}"] = {"tok_per_s": B * tm["decode_steps"] / tm["decode_s"],
-                        "ms_per_step": tm["decode_s"] * 1e3 / tm["decode_steps"],
-                        "prefill_tok_per_s": B * prompt_len / tm["prefill_s"]}
+        _, first = model.generate_graph(prompts, new_tokens + 1, return_first_logits=True, timings=tm)
+        step_s = tm["decode_s"] / tm["decode_steps"]
+        tw = {}
+        _, first_w = as_written.generate_graph(prompts, new_tokens + 1, return_first_logits=True, timings=tw)
+        # experts used per layer in a decode step: the routing of the first step's hidden states
+        used = []
+
+        def counting_moe(i, h):
+            idx, _ = routed_ids(kernels, h, w["layers"][i]["router"])
+            used.append(int((torch.bincount(idx.flatten().long(), minlength=s.experts) > 0).sum()))
+            return kernels.moe_layer(h, *layers[i], s.top_k, s.norm_topk_prob)
+
+        probe = D.Decoder(s, w, moe=counting_moe, max_positions=cap, attention="torch")
+        cache = D.KVCache(s, B, prompt_len + 4, torch.float16, dev)
+        nxt = probe.forward(tokens, cache)[:, -1].argmax(-1)
+        del used[:]
+        probe.forward(nxt[:, None], cache)
+        kv_bytes = s.layers * B * 2 * s.kv_heads * s.head_dim * (prompt_len + new_tokens / 2) * 2
+        step_bytes = sum(used) * EXPERT_BYTES + attn_bytes + router_bytes + head_bytes + kv_bytes
+        del cache, probe
+        # the MoE layers alone at this batch size: a stream of the 16 layers' calls
+        hB = hidden(B).to(dev)
+        moe_ms, _ = time_layer(kernels, hB, layers, "auto", 10 * s.layers, s.layers, spin=False)
+        # the per-expert loop in the hook on the same prompts: the first token must be its top-1
+        ref_first = loop_model.forward(tokens)[:, -1]
+        agree = first.argmax(-1) == ref_first.argmax(-1)
+        agree_w = first_w.argmax(-1) == ref_first.argmax(-1)
+        out[f"b{B}"] = {"tok_per_s": B / step_s, "ms_per_step": step_s * 1e3,
+                        "prefill_tok_per_s": B * prompt_len / tm["prefill_s"],
+                        "attention_torch_tok_per_s": B * tw["decode_steps"] / tw["decode_s"],
+                        "attention_torch_ms_per_step": tw["decode_s"] * 1e3 / tw["decode_steps"],
+                        "experts_used_per_layer_mean": sum(used) / len(used), "bytes_per_step": step_bytes,
+                        "roofline_tok_per_s": B * HBM_PEAK_GBS * 1e9 / step_bytes,
+                        "roofline_frac": step_bytes / (HBM_PEAK_GBS * 1e9) / step_s,
+                        "attention_torch_roofline_frac": step_bytes / (HBM_PEAK_GBS * 1e9) / (tw["decode_s"] / tw["decode_steps"]),
+                        "moe_ms_per_step": moe_ms * s.layers, "moe_share_of_step": moe_ms * s.layers / (step_s * 1e3),
+                        "moe_share_of_attention_torch_step": moe_ms * s.layers / (tw["decode_s"] * 1e3 / tw["decode_steps"]),
+                        "top1_rows_identical_to_loop_hook": int(agree.sum()),
+                        "attention_torch_top1_rows_identical_to_loop_hook": int(agree_w.sum()), "rows": B,
+                        "first_logits_max_abs_diff_vs_loop_hook": (first.float() - ref_first.float()).abs().max().item()}
     return out
 
 
@@ -142,92 +387,35 @@ def run_default(args):
     h = h_cpu.to(dev)
     mode = args.mode
 
-    def step(j):
-        router, gu, dn = layers[j % len(layers)]
-        return kernels.moe_layer(h, router, gu, dn, TOPK, False, mode)
-
-    # experts that receive a token, per layer (the metric's numerator)
-    used = []
-    for router, gu, dn in layers:
-        idx, _ = kernels.route(h, router, TOPK, False)
-        used.append(int((torch.bincount(idx.flatten().long(), minlength=E) > 0).sum()))
-
-    # The clocks of an idle GPU take some milliseconds of work to come up (20 launches after an
-    # idle gap run several per cent slower than the same launches in a long stream), so the GPU
-    # is kept busy for SPIN_UP_MS with the same layer calls before the warm-up steps; nothing of
-    # it is timed.
-    spin_until = time.perf_counter() + SPIN_UP_MS / 1e3
-    while time.perf_counter() < spin_until:
-        for j in range(10):
-            step(j)
-        torch.cuda.synchronize()
-    for j in range(args.warmup):
-        step(j)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for j in range(args.steps):
-        step(j)
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ms_per_step = wall * 1e3 / args.steps
+    # ---- the headline: exactly `steps` layer calls after `warmup`, in a stream
+    used = experts_used(kernels, h, layers)
+    ms_per_step, ev_med = time_layer(kernels, h, layers, mode, args.steps, args.warmup)
     used_mean = sum(used[j % len(layers)] for j in range(args.steps)) / args.steps
     value = used_mean * EXPERT_BYTES / (ms_per_step / 1e3) / 1e9
+    value_ev = used[0] * EXPERT_BYTES / (ev_med / 1e3) / 1e9
 
-    # the same layer call timed with one event pair per call (the reference's method, median)
-    ev = event_times(lambda: step(0), 20)
-    ev_med = statistics.median(ev)
+    # ---- the dominant kernel of this size
+    roof, roof_down = projection_rooflines(kernels, N, layers, mode, args.steps, args.warmup)
 
-    # dominant kernel: the gate/up projection, one event pair per launch on the launch stream
-    router, gu, dn = layers[0]
-    idx, w = kernels.route(h, router, TOPK, False)
-    counts, offsets, token, wsorted, pos_of = kernels.ext().sort_by_expert(idx, w, E)
-    M = idx.numel()
-    use_gemv = (mode if mode != "auto" else kernels._auto(N, M, E)) == "gemv"
-    rot = []
-    for r_, g_, d_ in layers:
-        i_, w_ = kernels.route(h, r_, TOPK, False)
-        s_ = kernels.ext().sort_by_expert(i_, w_, E)
-        rot.append((g_, s_[1], s_[2]))
-    calls = [0]
-    n_layers_rot = len(layers)
-
-    def gate_up():
-        g_, off_, tok_ = rot[calls[0] % len(rot)]
-        calls[0] += 1
-        if use_gemv:
-            return kernels.ext().grouped_gemv(h, tok_, g_, off_, M, True, None, N)
-        return kernels.ext().grouped_gemm(h, tok_, g_, off_, None, 0, M, True, None)
-
-    for _ in range(max(3, args.warmup)):
-        gate_up()
-    calls[0] = 0
-    group = 10
-    kt = stream_times(gate_up, max(args.steps, 20), group)
-    k_ms = sum(kt) / len(kt)
-    launches = len(kt) * group
-    used_k = sum(used[j % n_layers_rot] for j in range(launches)) / launches
-    if use_gemv or M // E < 300:
-        alg = used_k * 2 * H * I * 2                      # gate and up rows of every used expert, once
-        roof = {"bound": "hbm", "achieved": alg / (k_ms / 1e3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s"}
-    else:
-        alg = M * 4 * H * I                                # 2 * rows * 2I * H flops
-        roof = {"bound": "mfma", "achieved": alg / (k_ms / 1e3) / 1e12, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s"}
-    roof["frac"] = roof["achieved"] / roof["peak"]
-    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(N)
-    roof["kernel"] = "gemv_kernel<swiglu> (gate/up projection)" if use_gemv else "grouped_gemm<swiglu> (gate/up projection)"
-    roof["us_per_launch"] = k_ms * 1e3
-    roof["algorithmic_per_launch"] = alg
-
+    whole = not args.no_cpu and N == 8 and mode == "auto"   # the default run reports the whole metric
     cpu = None if args.no_cpu else cpu_loop_baseline(h_cpu, *cpu_layers[0], used[0])
-    n_layers = len(layers)
-    decode = None
-    if not args.no_cpu and N == 8 and mode == "auto":   # the default run reports the whole metric
-        del layers, rot, router, gu, dn
+    sizes = prefill = gpu_loop = decode = None
+    if whole:
+        sizes = {str(n): layer_record(kernels, n, layers, "auto", 100, 10) for n in DECODE_SIZES}
+        big = max(PREFILL_SIZES)
+        prefill = layer_record(kernels, big, layers, "gemm", 50, 5)
+        prefill["roofline"], prefill["down_projection"] = projection_rooflines(kernels, big, layers, "gemm", 100, 5)
+        prefill["other_sizes"] = {str(n): layer_record(kernels, n, layers, "gemm", 50, 5) for n in PREFILL_SIZES if n != big}
+        gpu_loop = gpu_loop_baseline(layers)
+        n_layers = len(layers)
+        del layers
         torch.cuda.empty_cache()
         try:
             decode = decode_rates()
         except Exception as exc:  # the layer figures above stand on their own
             decode = {"error": f"{type(exc).__name__}: {exc}"}
+    else:
+        n_layers = len(layers)
 
     line = {
         "metric": "OLMoE MoE-layer expert-weight GB/s", "value": value, "unit": "GB/s", "n_gpus": 1,
@@ -237,12 +425,16 @@ def run_default(args):
         "config": {"workload": f"olmoe_moe_layer_{'decode' if N <= 64 else 'prefill'}_{N}tok", "tokens": N,
                    "experts": E, "top_k": TOPK, "hidden": H, "expert_width": I, "mode": mode,
                    "layers_rotated": n_layers, "experts_used_mean": used_mean, "spin_up_ms": SPIN_UP_MS},
-        "us_per_layer": ms_per_step * 1e3, "us_per_layer_event_median": ev_med * 1e3,
-        "frac_of_hbm_peak": value / HBM_PEAK_GBS,
+        "timing": TIMING,
+        "us_per_layer": ms_per_step * 1e3, "frac_of_hbm_peak": value / HBM_PEAK_GBS,
+        "value_event_median": value_ev, "us_per_layer_event_median": ev_med * 1e3,
+        "frac_of_hbm_peak_event_median": value_ev / HBM_PEAK_GBS,
         "tflops": N * TOPK * 6 * H * I / (ms_per_step / 1e3) / 1e12,
-        "vs_baseline_note": "published figure is the reference's on one Tesla T4 (320 GB/s)",
+        "vs_baseline_note": "published figure is the reference's on one Tesla T4 (320 GB/s), event-timed single calls; "
+                            "`value` is the stream-of-layers figure, `value_event_median` the like-for-like one",
         "gpu": torch.cuda.get_device_name(0),
-        "roofline": roof, "cpu_baseline": cpu, "decode": decode,
+        "roofline": roof, "down_projection": roof_down, "cpu_baseline": cpu, "gpu_loop_fp16": gpu_loop,
+        "decode_sizes": sizes, "prefill": prefill, "decode": decode,
     }
     print(json.dumps(line), flush=True)
 
