@@ -1,8 +1,8 @@
 // grouped_gemm: the prefill path. Every expert's slice of the sorted rows goes through that
 // expert's weights on fp16 MFMA tiles, all experts in one launch. Three tiles, chosen by the
 // host from the mean rows per expert: 64 or 128 rows (gemm_kernel, below) while the launch is
-// mostly a stream over the weights, 256 rows (gemm_big_kernel, further down) once it is bound
-// by the MFMAs.
+// mostly a stream over the weights, 256 rows (gemm_stream_kernel, further down) once it is
+// bound by the MFMAs and by what a compute unit can pull through its L1.
 //
 // gemm_kernel. Tile: 64*MI rows x 256 weight rows (MI = 1 or 2), K in slices of 64, 4 wavefronts, each computing
 // all of the tile's rows x 64 weight rows as (2*MI) x 2 v_mfma_f32_32x32x16_f16 blocks with fp32
@@ -274,13 +274,16 @@ gemm_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const 
 
 // ---------------------------------------------------------------------------------------------
 // The tile for many rows per expert: 256 rows x 256 weight rows, 8 wavefronts (2 x 4, each 128
-// rows x 64 weight rows), one workgroup per CU.
+// rows x 64 weight rows), one workgroup per CU, and that workgroup stays: it walks its share of
+// the tile list as one stream.
 //
 // A 128-row tile asks the CU for 48 KB of operands per 1024 MFMA cycles, more than the path
-// from L2 delivers (about 44 B per clock per CU for rows of 128 bytes, half of that for rows
-// of 64), and moving them through registers into LDS costs more LDS write cycles than the
-// MFMAs take. This tile halves the bytes per flop and lets the memory pipeline write LDS
-// itself (buffer loads with the LDS modifier): no staging registers and no ds_write.
+// from L2 delivers, and moving them through registers into LDS costs more LDS write cycles than
+// the MFMAs take. This tile halves the bytes per flop and lets the memory pipeline write LDS
+// itself (buffer loads with the LDS modifier): no staging registers and no ds_write. Even so a
+// full tile's 2 MB of operands take a CU about as long to pull in as its MFMAs take (a loop of
+// the loads alone runs at 25 B per clock and CU: 85 thousand cycles against 65 thousand of
+// MFMAs), so nothing else may stand in front of either.
 //
 // All 160 KB of LDS are operand slices of 32 KB: two of the rows, three of the weight rows.
 // The rows of a tile are shared by all its column tiles and mostly hit in L2; the weights are
@@ -291,6 +294,20 @@ gemm_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const 
 // wavefront has read all of slice i, so the MFMAs of the last step run while the first
 // operands of slice i + 1 are read and the loads of rows i + 2 and weights i + 3 go out, one
 // at a time between the MFMAs, into the buffers that slice i has just left.
+//
+// The slices of a workgroup's tiles form one sequence: in a tile's last iterations the loads
+// that run ahead already belong to the next tile, so its first slices are in LDS when the
+// epilogue of this one is done. What a tile launched as a workgroup of its own pays in front of
+// an idle MFMA pipe (the lookup in the tile list, the row numbers, the latency of the first
+// loads, the launch of the workgroup: 6 to 9 of 55 microseconds) is paid once per launch here.
+// A tile's row numbers are read through the scalar cache, whose counter the vector loads in
+// flight do not share: those are counted by hand (below) and must never be waited for by a
+// load the compiler knows about.
+//
+// Which tiles a workgroup takes is fixed by its number (no queue, no atomics): the list is
+// ordered tallest tile first and dealt back and forth, consecutive places to workgroups of one
+// XCD, and when the tiles do not divide evenly the workgroups with one tile fewer get the
+// tallest ones (see the kernel).
 //
 // One such load writes the 64 lanes' 16 bytes to 1 KB of consecutive LDS: 8 unpadded rows of
 // 128 bytes. Which 16 bytes of its row a lane fetches is therefore chosen so that the operand
@@ -318,7 +335,10 @@ __device__ __forceinline__ int4_t buffer_descriptor(const void* base, unsigned b
 }
 
 // 16 bytes per lane from buffer offset voffset + soffset to LDS address lds_addr + 16 * lane.
-// Only voffset is checked against the size of the buffer.
+// Only voffset is checked against the size of the buffer. The LDS address travels in m0, which
+// the statement declares as clobbered; the compiler reserves m0 and warns about that on principle.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
 __device__ __forceinline__ void load_to_lds(int4_t rsrc, unsigned voffset, unsigned soffset, unsigned lds_addr) {
   // the descriptor, the slice offset and the LDS address are the same in every lane; say so
 #pragma unroll
@@ -333,242 +353,347 @@ __device__ __forceinline__ void load_to_lds(int4_t rsrc, unsigned voffset, unsig
       : "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset)
       : "memory", "m0");
 }
+#pragma clang diagnostic pop
 
-// WN wavefronts side by side over the weight rows, two over the rows: 2 x 4 wavefronts of 128 rows x
-// 64 weight rows, or 2 x 2 of 128 x 128, which read a third less from LDS per MFMA and have a
-// SIMD each.
-template <int WN, bool SWIGLU, bool SCALE>
-__global__ void __launch_bounds__(2 * WN * WAVE, 1)
-gemm_big_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const half_t* __restrict__ B,
-                const int* __restrict__ offsets, int E, int Nout, int K, const half_t* __restrict__ scale,
-                half_t* __restrict__ C, int ncol_tiles) {
-  constexpr int BM = BIG_BM;
+template <int EPL>
+struct ExpertTable {
+  int first[EPL], count[EPL], tiles[EPL], lo[EPL];  // lane x holds experts x, x + 64, ...
+};
+
+struct StreamTile {
+  int e, row0, row_end, n0;
+  unsigned b_lo, b_hi;   // address of the expert's matrix
+  int rot;
+  bool valid;
+};
+
+template <bool SWIGLU, bool SCALE, int EPL>
+__global__ void __launch_bounds__(512, 1)
+gemm_stream_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const half_t* __restrict__ B,
+                   const int* __restrict__ offsets, int E, int M, int Nout, int K, const half_t* __restrict__ scale,
+                   half_t* __restrict__ C, int ncol_tiles) {
+  constexpr int BM = BIG_BM, WN = 4;
   constexpr int WAVES = 2 * WN, THREADS = WAVES * WAVE;
-  constexpr int NB = BW / (32 * WN);                    // 32-row weight blocks per wavefront
-  constexpr int LOADS = BIG_A_BYTES / (THREADS * 16);   // per thread, slice and operand
+  constexpr int NB = BW / (32 * WN);
+  constexpr int LOADS = BIG_A_BYTES / (THREADS * 16);
   __shared__ __attribute__((aligned(1024))) char lds[BIG_A_STAGES * BIG_A_BYTES + BIG_B_STAGES * BIG_B_BYTES];
-  static_assert(sizeof(lds) == 160 * 1024, "the whole LDS of a CU");
-
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  int e, row0, row_end, col_tile;
-  // the tile lookup borrows the first bytes of the operand buffers
-  if (!find_tile<BM>(offsets, E, ncol_tiles, reinterpret_cast<int*>(lds), e, row0, row_end, col_tile)) return;
-  __syncthreads();  // everyone has read the lookup's result before loads overwrite it
-  const int nrows = min(BM, row_end - row0);
-
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   constexpr int COLS = SWIGLU ? BW / 2 : BW;
-  const int n0 = col_tile * COLS;
   const int Nfull = SWIGLU ? 2 * Nout : Nout;
-  const half_t* Be = B + (size_t)e * Nfull * K;
-
-  // ---- loader: load q of wavefront w fills LDS rows 8 * (WAVES * q + w) .. + 8, of the tile's rows
-  // and of its weight rows; lane l brings row l / 8 of them, and of that row the chunk that
-  // belongs at position l % 8
   constexpr unsigned OUT_OF_RANGE = 0x80000000u;
-  const int4_t arsrc = buffer_descriptor(A, 0x7fffffffu);
-  const int4_t brsrc = buffer_descriptor(Be, (unsigned)((size_t)Nfull * K * 2));
-  unsigned oa[LOADS], ob[LOADS];
-#pragma unroll
-  for (int q = 0; q < LOADS; ++q) {
-    const int r = 8 * (WAVES * q + wave) + (lane >> 3);
-    const unsigned chunk = (unsigned)((lane & 7) ^ ((r >> 1) & 7));
-    const int src = r < nrows ? (a_rows ? a_rows[row0 + r] : row0 + r) : 0;
-    oa[q] = r < nrows ? ((unsigned)src * (unsigned)K + chunk * 8u) * 2u : OUT_OF_RANGE;
-    int wr, col;
-    if (SWIGLU) {
-      col = n0 + (r & (COLS - 1));
-      wr = r < COLS ? col : Nout + col;
-    } else {
-      col = n0 + r;
-      wr = col;
-    }
-    ob[q] = col < Nout ? ((unsigned)wr * (unsigned)K + chunk * 8u) * 2u : OUT_OF_RANGE;
-  }
   const int nk = K / BIG_BK;
-  const int rot = K % 2048 == 0 ? (e * 5) % nk : 0;  // the K slice this expert's tiles start at (see gemm_kernel)
-  // byte offset of the kt-th slice this tile visits (kt < nk + 3)
-  auto slice_offset = [&](int kt) {
-    int at = kt + rot;
-    while (at >= nk) at -= nk;
-    return (unsigned)at * (BIG_BK * 2);
+
+  // ---- the tile list: per expert ceil(n / 256) row tiles of equal height, each with its column
+  // tiles (the row tiles of one column tile adjacent); every wavefront keeps the table in registers
+  ExpertTable<EPL> tb;
+  int cls[EPL];   // 32-row blocks in one of the expert's tiles: what a tile costs
+#pragma unroll
+  for (int s = 0; s < EPL; ++s) {
+    const int x = s * WAVE + lane;
+    const int f = x < E ? offsets[x] : 0, l = x < E ? offsets[x + 1] : 0;
+    tb.first[s] = f;
+    tb.count[s] = l - f;
+    tb.tiles[s] = (l - f + BM - 1) / BM;
+    cls[s] = tb.tiles[s] ? (((l - f + tb.tiles[s] - 1) / tb.tiles[s] + 31) >> 5) : 0;
+    tb.lo[s] = 0;
+  }
+  // The list is ordered by tile height, tallest first (experts of one height in their own order),
+  // and dealt to the workgroups back and forth, so that a workgroup with one tile fewer than its
+  // neighbour has the taller ones.
+  int run = 0;
+  for (int c = BM / 32; c >= 1; --c) {
+    bool present = false;
+#pragma unroll
+    for (int s = 0; s < EPL; ++s) present |= __ballot(cls[s] == c) != 0;
+    if (!present) continue;
+#pragma unroll
+    for (int s = 0; s < EPL; ++s) {
+      const int mine = cls[s] == c ? tb.tiles[s] * ncol_tiles : 0;
+      const int inc = wave_inclusive_scan(mine, lane);
+      if (cls[s] == c) tb.lo[s] = run + inc - mine;
+      run += __shfl(inc, WAVE - 1, WAVE);
+    }
+  }
+  const int total = __builtin_amdgcn_readfirstlane(run);
+  // consecutive places of the list go to workgroups of one XCD (workgroups are dealt round-robin
+  // to the XCDs): neighbours share rows or weights and meet in that XCD's L2
+  const int G = gridDim.x;
+  const int place = (blockIdx.x % XCDS) * (G / XCDS) + blockIdx.x / XCDS;
+  // With T tiles for G workgroups, T = q * G + rem, rem workgroups must take q + 1 tiles and the
+  // other G - rem take q. The latter get the tallest q * (G - rem) tiles of the list, so that four
+  // tall tiles stand against five lower ones; inside each group the tiles are dealt back and
+  // forth over full rounds, which evens out what is left of the difference in height.
+  const int q_tiles = total / G, rem = total - q_tiles * G;
+  const int n_short = rem ? G - rem : 0;                 // workgroups with q tiles
+  const bool is_short = place < n_short;
+  const int group = is_short ? n_short : G - n_short, seat = is_short ? place : place - n_short;
+  const int group_first = is_short ? 0 : q_tiles * n_short, group_rounds = is_short || !rem ? q_tiles : q_tiles + 1;
+  auto logical_of = [&](int r) {
+    return r < group_rounds ? group_first + r * group + ((r & 1) ? group - 1 - seat : seat) : total;
   };
+  const int list_end = total;
+  const int4_t arsrc = buffer_descriptor(A, 0x7fffffffu);
+
+  // per-lane offsets of the tile being loaded; the tile being computed keeps what its epilogue needs
+  auto lookup = [&](int logical, StreamTile& t, unsigned (&oa)[LOADS], unsigned (&ob)[LOADS]) {
+    t.valid = logical < list_end;
+    int e = 0, first = 0, count = 0, tiles = 1, lo = 0;
+    if (t.valid) {
+#pragma unroll
+      for (int s = 0; s < EPL; ++s) {
+        const uint64_t hit = __ballot(logical >= tb.lo[s] && logical < tb.lo[s] + tb.tiles[s] * ncol_tiles);
+        if (hit) {
+          const int src = __builtin_ctzll(hit);
+          e = s * WAVE + src;
+          first = __builtin_amdgcn_readlane(tb.first[s], src);
+          count = __builtin_amdgcn_readlane(tb.count[s], src);
+          tiles = __builtin_amdgcn_readlane(tb.tiles[s], src);
+          lo = __builtin_amdgcn_readlane(tb.lo[s], src);
+        }
+      }
+    }
+    const int within = logical - lo;
+    const int col = within / tiles, rt = within - col * tiles;
+    const int height = ((count + tiles - 1) / tiles + 31) & ~31;
+    t.e = e;
+    t.row0 = first + rt * height;
+    t.row_end = t.valid ? min(t.row0 + height, first + count) : t.row0;
+    t.n0 = col * COLS;
+    const uint64_t be = (uint64_t)(B + (size_t)e * Nfull * K);
+    t.b_lo = (unsigned)be;
+    t.b_hi = (unsigned)(be >> 32) & 0xffffu;
+    t.rot = K % 2048 == 0 ? (e * 5) % nk : 0;
+    const int nrows = t.row_end - t.row0;
+#pragma unroll
+    for (int q = 0; q < LOADS; ++q) {
+      const int rbase = 8 * (WAVES * q + wave);     // the 8 rows this load brings
+      const int r = rbase + (lane >> 3);
+      const unsigned chunk = (unsigned)((lane & 7) ^ ((r >> 1) & 7));
+      int src = t.row0 + r;
+      if (a_rows) {
+        // row numbers through the scalar path (its own counter: the vector loads in flight are
+        // counted by hand and must not be waited for here)
+        int picked = 0;
+#pragma unroll
+        for (int jj = 0; jj < 8; ++jj) {
+          const int v = a_rows[__builtin_amdgcn_readfirstlane(min(t.row0 + rbase + jj, M - 1))];
+          picked = (lane >> 3) == jj ? v : picked;
+        }
+        src = picked;
+      }
+      oa[q] = r < nrows ? ((unsigned)src * (unsigned)K + chunk * 8u) * 2u : OUT_OF_RANGE;
+      int wr, colw;
+      if (SWIGLU) {
+        colw = t.n0 + (r & (COLS - 1));
+        wr = r < COLS ? colw : Nout + colw;
+      } else {
+        colw = t.n0 + r;
+        wr = colw;
+      }
+      ob[q] = (t.valid && colw < Nout) ? ((unsigned)wr * (unsigned)K + chunk * 8u) * 2u : OUT_OF_RANGE;
+    }
+  };
+
   const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) char*)lds;
   const unsigned wave_base = __builtin_amdgcn_readfirstlane(lds_base + wave * 1024);
-  // load q (0 .. LOADS - 1) of the rows, or of the weight rows, of slice kt into buffer `stage`; past K
-  // it is still issued, out of range (only the per-lane offset is checked), and moves nothing
-  auto issue_rows = [&](int kt, int stage, int q) {
-    load_to_lds(arsrc, kt < nk ? oa[q] : OUT_OF_RANGE, slice_offset(kt), wave_base + stage * BIG_A_BYTES + q * (WAVES * 1024));
+  const unsigned b_bytes = (unsigned)((size_t)Nfull * K * 2);
+
+  StreamTile cur, nxt;
+  unsigned oa_c[LOADS], ob_c[LOADS], oa_n[LOADS], ob_n[LOADS];
+  lookup(logical_of(0), cur, oa_c, ob_c);
+  if (!cur.valid) return;
+  nxt = cur;   // until the second tile is known, nothing of the stream refers to it
+#pragma unroll
+  for (int q = 0; q < LOADS; ++q) {
+    oa_n[q] = oa_c[q];
+    ob_n[q] = ob_c[q];
+  }
+  int round = 1;
+
+  // load q of stream slice p (counted from the current tile's first slice; p >= nk is the next tile's)
+  auto issue_rows = [&](int p, int stage, int q) {
+    const bool later = p >= nk;
+    const int rot_c = cur.rot, rot_n = nxt.rot;
+    int at = later ? p - nk + rot_n : p + rot_c;
+    at = at >= nk ? at - nk : at;
+    const unsigned vc = oa_c[q], vn = oa_n[q];
+    load_to_lds(arsrc, later ? vn : vc, (unsigned)at * (BIG_BK * 2), wave_base + stage * BIG_A_BYTES + q * (WAVES * 1024));
   };
-  auto issue_weights = [&](int kt, int stage, int q) {
-    load_to_lds(brsrc, kt < nk ? ob[q] : OUT_OF_RANGE, slice_offset(kt),
+  auto issue_weights = [&](int p, int stage, int q) {
+    const bool later = p >= nk;
+    const int rot_c = cur.rot, rot_n = nxt.rot;
+    int at = later ? p - nk + rot_n : p + rot_c;
+    at = at >= nk ? at - nk : at;
+    const unsigned vc = ob_c[q], vn = ob_n[q];
+    const unsigned lo_c = cur.b_lo, lo_n = nxt.b_lo, hi_c = cur.b_hi, hi_n = nxt.b_hi;
+    int4_t rsrc;
+    rsrc[0] = (int)(later ? lo_n : lo_c);
+    rsrc[1] = (int)(later ? hi_n : hi_c);
+    rsrc[2] = (int)b_bytes;
+    rsrc[3] = 0x00020000;
+    load_to_lds(rsrc, later ? vn : vc, (unsigned)at * (BIG_BK * 2),
                 wave_base + BIG_A_STAGES * BIG_A_BYTES + stage * BIG_B_BYTES + q * (WAVES * 1024));
   };
 
-  // ---- wavefront tile: the 32-row blocks wm, wm + 2, wm + 4, wm + 6 (so that the two wavefronts
-  // that share weight rows split a short tile's live blocks evenly), weight rows
-  // brow[j] .. + 32 (with SwiGLU the first
-  // half of them gate rows and the second half the up rows of the same columns)
   const int wm = wave / WN, wn = wave % WN;
   const int l32 = lane & 31;
   int brow[NB];
 #pragma unroll
   for (int j = 0; j < NB; ++j)
     brow[j] = SWIGLU ? (j < NB / 2 ? 0 : COLS) + wn * (NB / 2 * 32) + (j % (NB / 2)) * 32 : wn * (NB * 32) + j * 32;
-  // byte offset inside a row of K-step s (16 halves = chunks 2s and 2s + 1; the upper 32 lanes
-  // take the second); every 32-row block starts at a multiple of 32, so the swizzle depends on
-  // the lane alone
   int koff[BIG_STEPS];
 #pragma unroll
   for (int s = 0; s < BIG_STEPS; ++s) koff[s] = (((2 * s + (lane >> 5)) ^ ((l32 >> 1) & 7)) * 16);
-
-  float16_t acc[4][NB];
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int j = 0; j < NB; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-
   const char* as = lds + (wm * 32 + l32) * BIG_ROW_BYTES;
   const char* bs = lds + BIG_A_STAGES * BIG_A_BYTES + l32 * BIG_ROW_BYTES;
 
-  // The K loop for LIVE live row blocks (a compile-time count: the loop body is branch-free).
-  auto k_loop = [&](auto live_blocks) {
-    constexpr int LIVE = decltype(live_blocks)::value;
-    constexpr int READS = LIVE > 0 ? LIVE + NB : 0, MFMAS = NB * LIVE;
-    constexpr int PAIRS = READS < MFMAS ? READS : MFMAS;
-    half8_t xf[2][LIVE > 0 ? LIVE : 1], wf[2][NB];  // operands of even and odd K-steps
-    // operand r of K-step s of the slice whose rows start at byte sa and weights at sb: the
-    // weight blocks, then the row blocks
-    auto read = [&](int sa, int sb, int s, int r) {
-      if (r < NB) wf[s & 1][r] = *reinterpret_cast<const half8_t*>(bs + sb + brow[r] * BIG_ROW_BYTES + koff[s]);
-      else xf[s & 1][r - NB] = *reinterpret_cast<const half8_t*>(as + sa + (r - NB) * 64 * BIG_ROW_BYTES + koff[s]);
-    };
-    auto mfma = [&](int s, int m) {
-      const int i = m / NB, j = m % NB;
-      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[s & 1][j], xf[s & 1][i], acc[i][j], 0, 0, 0);
-    };
-    // issue order: rows 0, weights 0 | rows 1, weights 1 | weights 2; from then on rows i + 2
-    // and then weights i + 3, so that "slice i + 1 has landed" is always "all but the last LOADS"
+  // ---- fill the pipe for the first tile: rows 0, weights 0 | rows 1, weights 1 | weights 2
 #pragma unroll
-    for (int p = 0; p < 2; ++p) {
+  for (int p = 0; p < 2; ++p) {
 #pragma unroll
-      for (int q = 0; q < LOADS; ++q) issue_rows(p, p, q);
+    for (int q = 0; q < LOADS; ++q) issue_rows(p, p, q);
 #pragma unroll
-      for (int q = 0; q < LOADS; ++q) issue_weights(p, p, q);
-    }
+    for (int q = 0; q < LOADS; ++q) issue_weights(p, p, q);
+  }
 #pragma unroll
-    for (int q = 0; q < LOADS; ++q) issue_weights(2, 2, q);
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * LOADS) : "memory");  // slice 0 has landed
-    __syncthreads();
+  for (int q = 0; q < LOADS; ++q) issue_weights(2, 2, q);
+  // the second tile is looked up while the first tile's loads are on their way
+  lookup(logical_of(round++), nxt, oa_n, ob_n);
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * LOADS) : "memory");
+  __syncthreads();
+  int a_stage = 0, b_stage = 0;  // where the current tile's slice 0 is
+
+  float16_t acc[4][NB];
+  for (;;) {
 #pragma unroll
-    for (int r = 0; r < READS; ++r) read(0, 0, 0, r);
-    int a_stage = 0, b_stage = 0;  // where slice kt is
-    for (int kt = 0; kt < nk; ++kt) {
-      const int a_next = a_stage ^ 1, b_next = b_stage == BIG_B_STAGES - 1 ? 0 : b_stage + 1;
-      const int sa = a_stage * BIG_A_BYTES, sb = b_stage * BIG_B_BYTES;
-      // all steps but the last, each with the reads of the next step behind its MFMAs
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int s = 0; s < BIG_STEPS - 1; ++s) {
+      for (int j = 0; j < NB; ++j)
 #pragma unroll
-        for (int r = 0; r < READS; ++r) read(sa, sb, s + 1, r);
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    // On entry slice 0 of the current tile has landed and every wavefront knows it.
+    auto k_loop = [&](auto live_blocks) {
+      constexpr int LIVE = decltype(live_blocks)::value;
+      constexpr int READS = LIVE > 0 ? LIVE + NB : 0, MFMAS = NB * LIVE;
+      constexpr int PAIRS = READS < MFMAS ? READS : MFMAS;
+      half8_t xf[2][LIVE > 0 ? LIVE : 1], wf[2][NB];
+      auto read = [&](int sa, int sb, int s, int r) {
+        if (r < NB) wf[s & 1][r] = *reinterpret_cast<const half8_t*>(bs + sb + brow[r] * BIG_ROW_BYTES + koff[s]);
+        else xf[s & 1][r - NB] = *reinterpret_cast<const half8_t*>(as + sa + (r - NB) * 64 * BIG_ROW_BYTES + koff[s]);
+      };
+      auto mfma = [&](int s, int m) {
+        const int i = m / NB, j = m % NB;
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[s & 1][j], xf[s & 1][i], acc[i][j], 0, 0, 0);
+      };
 #pragma unroll
-        for (int m = 0; m < MFMAS; ++m) mfma(s, m);
-      }
+      for (int r = 0; r < READS; ++r) read(a_stage * BIG_A_BYTES, b_stage * BIG_B_BYTES, 0, r);
+      for (int kt = 0; kt < nk; ++kt) {
+        const int a_next = a_stage ^ 1, b_next = b_stage == BIG_B_STAGES - 1 ? 0 : b_stage + 1;
+        const int sa = a_stage * BIG_A_BYTES, sb = b_stage * BIG_B_BYTES;
 #pragma unroll
-      for (int s = 0; s < BIG_STEPS - 1; ++s) {
+        for (int s = 0; s < BIG_STEPS - 1; ++s) {
 #pragma unroll
-        for (int n = 0; n < PAIRS; ++n) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          for (int r = 0; r < READS; ++r) read(sa, sb, s + 1, r);
+#pragma unroll
+          for (int m = 0; m < MFMAS; ++m) mfma(s, m);
         }
-        if (READS > PAIRS) __builtin_amdgcn_sched_group_barrier(0x100, READS - PAIRS, 0);
-        if (MFMAS > PAIRS) __builtin_amdgcn_sched_group_barrier(0x008, MFMAS - PAIRS, 0);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-      // slice kt + 1 has landed (the weights of slice kt + 2 may be out) and this wavefront's
-      // reads of slice kt are complete
-      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(LOADS) : "memory");
-      __syncthreads();
-      // the last step in parts, each followed by one load: rows kt + 2, then weights kt + 3
 #pragma unroll
-      for (int part = 0; part < 2 * LOADS; ++part) {
+        for (int s = 0; s < BIG_STEPS - 1; ++s) {
 #pragma unroll
-        for (int r = 0; r < READS; ++r)
-          if (r * 2 * LOADS / (READS > 0 ? READS : 1) == part) read(a_next * BIG_A_BYTES, b_next * BIG_B_BYTES, 0, r);
-#pragma unroll
-        for (int m = 0; m < MFMAS; ++m)
-          if (m * 2 * LOADS / (MFMAS > 0 ? MFMAS : 1) == part) mfma(BIG_STEPS - 1, m);
+          for (int n = 0; n < PAIRS; ++n) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          }
+          if (READS > PAIRS) __builtin_amdgcn_sched_group_barrier(0x100, READS - PAIRS, 0);
+          if (MFMAS > PAIRS) __builtin_amdgcn_sched_group_barrier(0x008, MFMAS - PAIRS, 0);
+        }
         __builtin_amdgcn_sched_barrier(0);
-        if (part < LOADS) issue_rows(kt + 2, a_stage, part);
-        else issue_weights(kt + 3, b_stage, part - LOADS);
-        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(LOADS) : "memory");
+        __syncthreads();
+#pragma unroll
+        for (int part = 0; part < 2 * LOADS; ++part) {
+#pragma unroll
+          for (int r = 0; r < READS; ++r)
+            if (r * 2 * LOADS / (READS > 0 ? READS : 1) == part) read(a_next * BIG_A_BYTES, b_next * BIG_B_BYTES, 0, r);
+#pragma unroll
+          for (int m = 0; m < MFMAS; ++m)
+            if (m * 2 * LOADS / (MFMAS > 0 ? MFMAS : 1) == part) mfma(BIG_STEPS - 1, m);
+          __builtin_amdgcn_sched_barrier(0);
+          if (part < LOADS) issue_rows(kt + 2, a_stage, part);
+          else issue_weights(kt + 3, b_stage, part - LOADS);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        a_stage = a_next;
+        b_stage = b_next;
       }
-      a_stage = a_next;
-      b_stage = b_next;
+    };
+    const int nrows = cur.row_end - cur.row0;
+    const int live = ((nrows + 31) / 32 + 1 - wm) / 2;
+    switch (live) {
+      case 4: k_loop(std::integral_constant<int, 4>{}); break;
+      case 3: k_loop(std::integral_constant<int, 3>{}); break;
+      case 2: k_loop(std::integral_constant<int, 2>{}); break;
+      case 1: k_loop(std::integral_constant<int, 1>{}); break;
+      default: k_loop(std::integral_constant<int, 0>{}); break;
     }
-  };
-  const int live = ((nrows + 31) / 32 + 1 - wm) / 2;  // of the tile's live blocks, those this wavefront owns
-  switch (live) {
-    case 4: k_loop(std::integral_constant<int, 4>{}); break;
-    case 3: k_loop(std::integral_constant<int, 3>{}); break;
-    case 2: k_loop(std::integral_constant<int, 2>{}); break;
-    case 1: k_loop(std::integral_constant<int, 1>{}); break;
-    default: k_loop(std::integral_constant<int, 0>{}); break;
+    // ---- epilogue of the current tile (the next tile's first slices are in flight meanwhile)
+    const int chalf = (lane >> 5) * 4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = cur.row0 + (2 * i + wm) * 32 + l32;
+      if (row >= cur.row_end) continue;
+      const float sc_row = SCALE ? (float)scale[row] : 1.f;
+      half_t* crow = C + (size_t)row * Nout;
+      constexpr int NJ = SWIGLU ? NB / 2 : NB;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        const int cbase = cur.n0 + wn * (NJ * 32) + j * 32 + chalf;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int c0 = cbase + 8 * q;
+          half4_t o;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float v = acc[i][j][4 * q + r];
+            if (SWIGLU) o[r] = swiglu_f16(v, acc[i][SWIGLU ? j + NB / 2 : j][4 * q + r]);
+            else if (SCALE) o[r] = (half_t)((float)(half_t)v * sc_row);
+            else o[r] = (half_t)v;
+          }
+          if (c0 + 3 < Nout && (Nout & 3) == 0) {
+            *reinterpret_cast<half4_t*>(crow + c0) = o;
+          } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+              if (c0 + r < Nout) crow[c0 + r] = o[r];
+          }
+        }
+      }
+    }
+    if (!nxt.valid) break;
+    cur = nxt;
+#pragma unroll
+    for (int q = 0; q < LOADS; ++q) {
+      oa_c[q] = oa_n[q];
+      ob_c[q] = ob_n[q];
+    }
+    lookup(logical_of(round++), nxt, oa_n, ob_n);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no load may land in LDS after this workgroup has given it back
-
-  // ---- epilogue: acc element 4*q + r of block (i, j) is row i*32 + l32, column 8*q + 4*(lane/32) + r
-  const int chalf = (lane >> 5) * 4;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int row = row0 + (2 * i + wm) * 32 + l32;
-    if (row >= row_end) continue;
-    const float sc_row = SCALE ? (float)scale[row] : 1.f;
-    half_t* crow = C + (size_t)row * Nout;
-    constexpr int NJ = SWIGLU ? NB / 2 : NB;  // blocks of 32 output columns
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-      const int cbase = n0 + wn * (NJ * 32) + j * 32 + chalf;
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int c0 = cbase + 8 * q;
-        half4_t o;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const float v = acc[i][j][4 * q + r];
-          if (SWIGLU) o[r] = swiglu_f16(v, acc[i][SWIGLU ? j + NB / 2 : j][4 * q + r]);
-          else if (SCALE) o[r] = (half_t)((float)(half_t)v * sc_row);
-          else o[r] = (half_t)v;
-        }
-        if (c0 + 3 < Nout && (Nout & 3) == 0) {
-          *reinterpret_cast<half4_t*>(crow + c0) = o;
-        } else {
-#pragma unroll
-          for (int r = 0; r < 4; ++r)
-            if (c0 + r < Nout) crow[c0 + r] = o[r];
-        }
-      }
-    }
-  }
 }
 
-template <int WN>
-int launch_gemm_big(const half_t* a, const int32_t* a_rows, const half_t* b, const int32_t* offsets, int E, int rows,
-                    int Nout, int K, int swiglu, const half_t* s, half_t* c, hipStream_t st) {
+template <int EPL>
+int launch_gemm_stream(const half_t* a, const int32_t* a_rows, const half_t* b, const int32_t* offsets, int E, int rows,
+                       int Nout, int K, int swiglu, const half_t* s, half_t* c, hipStream_t st) {
   const int cols = swiglu ? BW / 2 : BW;
   const int ncol_tiles = (Nout + cols - 1) / cols;
-  const long max_row_tiles = rows / BIG_BM + (E < rows ? E : rows);
-  const long total = max_row_tiles * ncol_tiles;
-  if (total >= (1l << 31) - XCDS) return sy_fail(SY_ERR_ARG, "grouped_gemm: too many tiles");
-  const int per_xcd = (int)((total + XCDS - 1) / XCDS);
-  const int grid = per_xcd * XCDS;
+  const int grid = sy_compute_units() / XCDS * XCDS;
   if (swiglu)
-    gemm_big_kernel<WN, true, false><<<grid, 2 * WN * WAVE, 0, st>>>(a, a_rows, b, offsets, E, Nout, K, nullptr, c, ncol_tiles);
+    gemm_stream_kernel<true, false, EPL><<<grid, 512, 0, st>>>(a, a_rows, b, offsets, E, rows, Nout, K, nullptr, c, ncol_tiles);
   else if (s)
-    gemm_big_kernel<WN, false, true><<<grid, 2 * WN * WAVE, 0, st>>>(a, a_rows, b, offsets, E, Nout, K, s, c, ncol_tiles);
+    gemm_stream_kernel<false, true, EPL><<<grid, 512, 0, st>>>(a, a_rows, b, offsets, E, rows, Nout, K, s, c, ncol_tiles);
   else
-    gemm_big_kernel<WN, false, false><<<grid, 2 * WN * WAVE, 0, st>>>(a, a_rows, b, offsets, E, Nout, K, nullptr, c, ncol_tiles);
+    gemm_stream_kernel<false, false, EPL><<<grid, 512, 0, st>>>(a, a_rows, b, offsets, E, rows, Nout, K, nullptr, c, ncol_tiles);
   return sy_check_launch("grouped_gemm");
 }
 
@@ -614,9 +739,13 @@ extern "C" SY_API int sy_grouped_gemm(const void* A, const int32_t* a_rows, cons
   const half_t* b = (const half_t*)B;
   const half_t* s = (const half_t*)scale;
   half_t* c = (half_t*)C;
-  // measured on 64 experts, 2048 x 1024: the 256-row tile wins from about 128 rows per expert on
-  const int tile = typical <= 64 ? 64 : (typical <= 128 || K % BIG_BK) ? 128 : 256;
-  if (tile == 256) return launch_gemm_big<4>(a, a_rows, b, offsets, E, rows, Nout, K, swiglu, s, c, (hipStream_t)stream);
+  // measured on 64 experts, 2048 x 1024: the 256-row tile wins from about 128 rows per expert on.
+  // Its loads run three slices ahead, into the next tile, so it wants four slices of K; its tile
+  // table is one or two experts per lane.
+  const bool stream_ok = K % BIG_BK == 0 && K / BIG_BK >= 4 && E <= 2 * WAVE;
+  const int tile = typical <= 64 ? 64 : (typical <= 128 || !stream_ok) ? 128 : 256;
+  if (tile == 256 && E <= WAVE) return launch_gemm_stream<1>(a, a_rows, b, offsets, E, rows, Nout, K, swiglu, s, c, (hipStream_t)stream);
+  if (tile == 256) return launch_gemm_stream<2>(a, a_rows, b, offsets, E, rows, Nout, K, swiglu, s, c, (hipStream_t)stream);
   if (tile == 64) return launch_gemm<1>(a, a_rows, b, offsets, E, rows, Nout, K, swiglu, s, c, (hipStream_t)stream);
   return launch_gemm<2>(a, a_rows, b, offsets, E, rows, Nout, K, swiglu, s, c, (hipStream_t)stream);
 }
