@@ -402,6 +402,9 @@ def run_default(args):
     sizes = prefill = gpu_loop = decode = None
     if whole:
         sizes = {str(n): layer_record(kernels, n, layers, "auto", 100, 10) for n in DECODE_SIZES}
+        for n in DECODE_SIZES:   # the decode configuration names the weight-stream kernel: time it where "auto" prefers the tiles
+            if sizes[str(n)]["mode"] != "gemv":
+                sizes[f"{n}_gemv"] = layer_record(kernels, n, layers, "gemv", 100, 10)
         big = max(PREFILL_SIZES)
         prefill = layer_record(kernels, big, layers, "gemm", 50, 5)
         prefill["roofline"], prefill["down_projection"] = projection_rooflines(kernels, big, layers, "gemm", 100, 5)

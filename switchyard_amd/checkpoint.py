@@ -2,22 +2,26 @@
 sharded set with model.safetensors.index.json) into the tensors the decoder and the MoE
 kernels take.
 
-Counterpart of the reference's switchyard/weights.py (:15-69) and switchyard/config.py
-(:27-48): the same dictionary comes back, {"embed", "final_norm", "lm_head", "layers": [one
+It fills the role of the reference's switchyard/weights.py (:36-69) and switchyard/config.py
+(:27-48) and returns the same dictionary, {"embed", "final_norm", "lm_head", "layers": [one
 dict per layer], "experts"}, with a layer's experts stacked as gate_up [E, 2I, H] (gate rows
 0..I-1, up rows I..2I-1) and down [E, H, I], each in nn.Linear layout (out x in, the reduced
 dimension contiguous). That is the layout the kernels stream, so nothing is transposed or
 repacked on the way in.
 
-Built for a GPU that holds the whole model: every stacked tensor is allocated once on the
-target device and each expert's matrices are copied from the file's mapping straight into
-their rows of it, so the host never holds a second copy of a layer (a layer of OLMoE-1B-7B is
-805 MB of experts; the reference stacks 128 host tensors per layer and then moves the stack).
-Files are read with safetensors only: nothing in a checkpoint is executed.
+The reader is destination-driven and makes one pass over the files. Every output tensor is
+allocated on the target device first; a table then says, for each tensor name a checkpoint may
+hold, which slice of which output it belongs in. The files are visited one after the other,
+each opened once and closed again, and every tensor with an entry in the table is copied from
+the file's mapping straight into its slice (the copy converts the type and crosses to the
+device), so the host never holds a second copy of anything: a layer of OLMoE-1B-7B is 805 MB
+of experts. Tensors without an entry (experts that were not asked for) are never read. Files
+are read with safetensors only: nothing in a checkpoint is executed.
 """
 
 import json
 import os
+from types import SimpleNamespace
 
 import torch
 from safetensors import safe_open
@@ -29,59 +33,68 @@ SINGLE = "model.safetensors"
 
 
 def shape_from_config(path):
-    """The decoder's Shape from `path`/config.json (reference: Config.load, config.py:27-48).
-    Returns (shape, tie_embeddings)."""
+    """(Shape, tie_word_embeddings) from `path`/config.json; the field names are those of a
+    transformers OlmoeConfig, which Shape.from_hf reads."""
     with open(os.path.join(path, "config.json")) as f:
-        c = json.load(f)
-    heads = c["num_attention_heads"]
-    rope = c.get("rope_parameters") or {}
-    shape = Shape(vocab=c["vocab_size"], hidden=c["hidden_size"], intermediate=c["intermediate_size"],
-                  layers=c["num_hidden_layers"], heads=heads, kv_heads=c.get("num_key_value_heads") or heads,
-                  head_dim=c.get("head_dim") or c["hidden_size"] // heads, experts=c["num_experts"],
-                  top_k=c["num_experts_per_tok"], norm_topk_prob=bool(c.get("norm_topk_prob", False)),
-                  rms_eps=c.get("rms_norm_eps", 1e-5), rope_theta=rope.get("rope_theta", c.get("rope_theta", 10000.0)),
-                  clip_qkv=c.get("clip_qkv"))
-    return shape, bool(c.get("tie_word_embeddings", False))
+        fields = json.load(f)
+    return Shape.from_hf(SimpleNamespace(**fields)), bool(fields.get("tie_word_embeddings", False))
 
 
-class Checkpoint:
-    """Name -> tensor over the files of one checkpoint directory; files are opened on first use
-    and stay mapped until close()."""
+def tensor_files(path):
+    """{file name: [tensor names in it]} for the checkpoint directory `path`."""
+    index = os.path.join(path, INDEX)
+    files = {}
+    if os.path.exists(index):
+        with open(index) as f:
+            for name, file in json.load(f)["weight_map"].items():
+                files.setdefault(file, []).append(name)
+    elif os.path.exists(os.path.join(path, SINGLE)):
+        with safe_open(os.path.join(path, SINGLE), "pt") as f:
+            files[SINGLE] = list(f.keys())
+    else:
+        raise FileNotFoundError(f"{path}: neither {INDEX} nor {SINGLE}")
+    return files
 
-    def __init__(self, path):
-        self.path = path
-        index = os.path.join(path, INDEX)
-        if os.path.exists(index):
-            with open(index) as f:
-                self.where = dict(json.load(f)["weight_map"])
-        elif os.path.exists(os.path.join(path, SINGLE)):
-            with safe_open(os.path.join(path, SINGLE), "pt") as f:
-                self.where = {k: SINGLE for k in f.keys()}
-        else:
-            raise FileNotFoundError(f"{path}: neither {INDEX} nor {SINGLE}")
-        self._open = {}
 
-    def has(self, name):
-        return name in self.where
+class _Slot:
+    """Where one checkpoint tensor goes: `out` is the slice of an output tensor it fills; with
+    `rows`, the tensor in the file is a stack and only those rows of it are taken."""
 
-    def get(self, name):
-        if name not in self.where:
-            raise KeyError(f"{self.path}: no tensor named {name}")
-        file = self.where[name]
-        if file not in self._open:
-            self._open[file] = safe_open(os.path.join(self.path, file), "pt")
-        return self._open[file].get_tensor(name)
+    def __init__(self, out, rows=None):
+        self.out, self.rows, self.filled = out, rows, False
 
-    def close(self):
-        self._open.clear()
+    def fill(self, name, get):
+        x = get(name)
+        want = tuple(self.out.shape[1:]) if self.rows is not None else tuple(self.out.shape)
+        have = tuple(x.shape[1:]) if self.rows is not None else tuple(x.shape)
+        if have != want or (self.rows is not None and max(self.rows, default=-1) >= x.shape[0]):
+            raise ValueError(f"{name}: shape {tuple(x.shape)} in the file, {want} "
+                             f"{'per expert ' if self.rows is not None else ''}by config.json")
+        self.out.copy_(x if self.rows is None else x[torch.tensor(self.rows, dtype=torch.long)])
+        self.filled = True
+
+
+def _expert_lists(shape, experts, experts_per_layer):
+    experts = list(range(shape.experts)) if experts is None else [int(e) for e in experts]
+    if experts_per_layer is None:
+        per_layer = [experts] * shape.layers
+    elif len(experts_per_layer) != shape.layers:
+        raise ValueError(f"experts_per_layer has {len(experts_per_layer)} entries for {shape.layers} layers")
+    else:
+        per_layer = [[int(e) for e in mine] for mine in experts_per_layer]
+    for i, mine in enumerate(per_layer):
+        bad = [e for e in mine if not 0 <= e < shape.experts]
+        if bad:
+            raise ValueError(f"layer {i}: experts {bad} outside 0..{shape.experts - 1}")
+    return experts, per_layer
 
 
 def load(path, shape=None, dtype=torch.float16, device="cuda", experts=None, experts_per_layer=None):
     """The weights of the checkpoint at `path` on `device` in `dtype`.
 
     `experts` (default: all) picks which experts are stacked, in that order; with
-    `experts_per_layer`, layer i stacks experts_per_layer[i] instead (reference:
-    weights.load, weights.py:36-69). The router keeps all its rows either way.
+    `experts_per_layer`, layer i stacks experts_per_layer[i] instead (the arguments of the
+    reference's weights.load, weights.py:36-38). The router keeps all its rows either way.
     Both the per-expert tensor names of published OLMoE checkpoints
     (`mlp.experts.<j>.gate_proj.weight` ...) and the stacked names newer transformers keeps in
     memory (`mlp.experts.gate_up_proj`, `mlp.experts.down_proj`) are understood."""
@@ -90,53 +103,60 @@ def load(path, shape=None, dtype=torch.float16, device="cuda", experts=None, exp
         shape, tied = shape_from_config(path)
     elif os.path.exists(os.path.join(path, "config.json")):
         tied = shape_from_config(path)[1]
-    ck = Checkpoint(path)
-    experts = list(range(shape.experts)) if experts is None else [int(e) for e in experts]
-    if experts_per_layer is not None and len(experts_per_layer) != shape.layers:
-        raise ValueError(f"experts_per_layer has {len(experts_per_layer)} entries for {shape.layers} layers")
-    I, H = shape.intermediate, shape.hidden
-
-    def t(name, want=None):
-        x = ck.get(name)
-        if want is not None and tuple(x.shape) != tuple(want):
-            raise ValueError(f"{name}: shape {tuple(x.shape)} in the file, {tuple(want)} by config.json")
-        return x.to(device=device, dtype=dtype).contiguous()
-
-    def into(dst, name):
-        x = ck.get(name)
-        if tuple(x.shape) != tuple(dst.shape):
-            raise ValueError(f"{name}: shape {tuple(x.shape)} in the file, {tuple(dst.shape)} by config.json")
-        dst.copy_(x)          # converts and crosses to the device in one step, into the stack's own rows
-
+    experts, per_layer = _expert_lists(shape, experts, experts_per_layer)
+    files = tensor_files(path)
+    present = {name for names in files.values() for name in names}
+    H, I = shape.hidden, shape.intermediate
     qd, kvd = shape.heads * shape.head_dim, shape.kv_heads * shape.head_dim
-    out = {"embed": t("model.embed_tokens.weight", (shape.vocab, H)), "final_norm": t("model.norm.weight", (H,))}
-    out["lm_head"] = out["embed"] if tied or not ck.has("lm_head.weight") else t("lm_head.weight", (shape.vocab, H))
-    layers = []
-    for i in range(shape.layers):
-        p = f"model.layers.{i}."
-        mine = experts if experts_per_layer is None else [int(e) for e in experts_per_layer[i]]
-        bad = [e for e in mine if not 0 <= e < shape.experts]
-        if bad:
-            raise ValueError(f"layer {i}: experts {bad} outside 0..{shape.experts - 1}")
-        gate_up = torch.empty(len(mine), 2 * I, H, dtype=dtype, device=device)
-        down = torch.empty(len(mine), H, I, dtype=dtype, device=device)
-        e = p + "mlp.experts."
-        if ck.has(e + "gate_up_proj"):
-            pick = torch.tensor(mine, dtype=torch.long)
-            gate_up.copy_(ck.get(e + "gate_up_proj")[pick])
-            down.copy_(ck.get(e + "down_proj")[pick])
+
+    def new(*dims):
+        return torch.empty(*dims, dtype=dtype, device=device)
+
+    # ---- every output, and the table from checkpoint names to their places in them
+    slots = {}
+    out = {"embed": new(shape.vocab, H), "final_norm": new(H), "layers": [], "experts": experts}
+    slots["model.embed_tokens.weight"] = _Slot(out["embed"])
+    slots["model.norm.weight"] = _Slot(out["final_norm"])
+    if tied or "lm_head.weight" not in present:
+        out["lm_head"] = out["embed"]
+    else:
+        out["lm_head"] = new(shape.vocab, H)
+        slots["lm_head.weight"] = _Slot(out["lm_head"])
+    plain = (("attn_norm", "input_layernorm.weight", (H,)), ("mlp_norm", "post_attention_layernorm.weight", (H,)),
+             ("wq", "self_attn.q_proj.weight", (qd, H)), ("wk", "self_attn.k_proj.weight", (kvd, H)),
+             ("wv", "self_attn.v_proj.weight", (kvd, H)), ("wo", "self_attn.o_proj.weight", (H, qd)),
+             ("q_norm", "self_attn.q_norm.weight", (qd,)), ("k_norm", "self_attn.k_norm.weight", (kvd,)),
+             ("router", "mlp.gate.weight", (shape.experts, H)))
+    for i, mine in enumerate(per_layer):
+        prefix = f"model.layers.{i}."
+        layer = {key: new(*dims) for key, _, dims in plain}
+        layer["gate_up"], layer["down"] = new(len(mine), 2 * I, H), new(len(mine), H, I)
+        for key, suffix, _ in plain:
+            slots[prefix + suffix] = _Slot(layer[key])
+        stacked = prefix + "mlp.experts.gate_up_proj"
+        if stacked in present:   # one tensor holds all experts: take the rows asked for
+            slots[stacked] = _Slot(layer["gate_up"], rows=mine)
+            slots[prefix + "mlp.experts.down_proj"] = _Slot(layer["down"], rows=mine)
         else:
             for row, j in enumerate(mine):
-                into(gate_up[row, :I], f"{e}{j}.gate_proj.weight")
-                into(gate_up[row, I:], f"{e}{j}.up_proj.weight")
-                into(down[row], f"{e}{j}.down_proj.weight")
-        layers.append(dict(
-            attn_norm=t(p + "input_layernorm.weight", (H,)), mlp_norm=t(p + "post_attention_layernorm.weight", (H,)),
-            wq=t(p + "self_attn.q_proj.weight", (qd, H)), wk=t(p + "self_attn.k_proj.weight", (kvd, H)),
-            wv=t(p + "self_attn.v_proj.weight", (kvd, H)), wo=t(p + "self_attn.o_proj.weight", (H, qd)),
-            q_norm=t(p + "self_attn.q_norm.weight", (qd,)), k_norm=t(p + "self_attn.k_norm.weight", (kvd,)),
-            router=t(p + "mlp.gate.weight", (shape.experts, H)), gate_up=gate_up, down=down))
-    ck.close()
-    out["layers"] = layers
-    out["experts"] = experts
+                # the same expert may be stacked twice; each row is a place of its own
+                for part, view in (("gate_proj", layer["gate_up"][row, :I]), ("up_proj", layer["gate_up"][row, I:]),
+                                   ("down_proj", layer["down"][row])):
+                    slots.setdefault(f"{prefix}mlp.experts.{j}.{part}.weight", []).append(_Slot(view))
+        out["layers"].append(layer)
+
+    # ---- one pass over the files
+    for file, names in files.items():
+        wanted = [name for name in names if name in slots]
+        if not wanted:
+            continue
+        with safe_open(os.path.join(path, file), "pt") as f:
+            for name in wanted:
+                places = slots[name]
+                for slot in places if isinstance(places, list) else [places]:
+                    slot.fill(name, f.get_tensor)
+    for name, places in slots.items():
+        for slot in places if isinstance(places, list) else [places]:
+            if not slot.filled:
+                raise KeyError(f"{path}: no tensor named {name}")
     return out

@@ -113,6 +113,53 @@ def _rotate(x, cos, sin):
     return x * cos + torch.cat([-x[..., half:], x[..., :half]], dim=-1) * sin
 
 
+class Span:
+    """The T positions a forward call appends to a cache (or a whole sequence without one).
+
+    real [B, T]       False where a row holds left padding
+    first, end        the cache slots the span occupies
+    seen [B]          real tokens of each row before the span
+    positions [B, T]  rotary position of each new token: its index among its row's real tokens
+    visible           [B, 1, T, end] attention mask: a query sees the slots at or before its own
+                      that hold a real token; a padding query, which would see nothing, sees
+                      itself (its output is never used, but its softmax must not be empty)."""
+
+    def __init__(self, tokens, cache, real=None):
+        B, T = tokens.shape
+        dev = tokens.device
+        self.real = torch.ones(B, T, dtype=torch.bool, device=dev) if real is None else real
+        self.first = cache.filled if cache is not None else 0
+        self.end = self.first + T
+        self.seen = cache.next_position if cache is not None else torch.zeros(B, dtype=torch.long, device=dev)
+        order = self.real.long().cumsum(1)                       # 1-based index among the row's real tokens
+        self.positions = (self.seen[:, None] + order - 1).clamp_(min=0)
+        if cache is not None:
+            cache.real[:, self.first:self.end] = self.real
+            slot_real = cache.real[:, :self.end]
+        else:
+            slot_real = self.real
+        query_slot = torch.arange(self.first, self.end, device=dev)[:, None]
+        slot = torch.arange(self.end, device=dev)[None, :]
+        sees = (slot <= query_slot)[None] & slot_real[:, None, :]
+        alone = ~sees.any(-1, keepdim=True)
+        self.visible = (sees | (alone & (slot == query_slot)[None]))[:, None]   # broadcast over heads
+
+    def commit(self, cache):
+        """The span now belongs to the cache."""
+        cache.filled = self.end
+        cache.next_position = self.seen + self.real.long().sum(1)
+
+
+def left_padded(prompts, device):
+    """Token lists of unequal length as one right-aligned batch: (tokens [B, P], real [B, P])."""
+    lengths = torch.tensor([len(p) for p in prompts])
+    width = int(lengths.max())
+    real = torch.arange(width)[None, :] >= (width - lengths)[:, None]
+    tokens = torch.zeros(len(prompts), width, dtype=torch.long)
+    tokens[real] = torch.tensor([t for p in prompts for t in p], dtype=torch.long)   # row by row, in order
+    return tokens.to(device), real.to(device)
+
+
 class KVCache:
     """Keys and values of every layer, [B, kv_heads, capacity, head_dim], allocated once.
     `filled` positions are in use; `real[b, p]` is False where batch row b holds left padding."""
@@ -154,47 +201,30 @@ class Decoder:
         L = self.w["layers"][i]
         return kernels.moe_layer(h, L["router"], L["gate_up"], L["down"], self.s.top_k, self.s.norm_topk_prob)
 
-    def _attend(self, i, x, positions, mask, cache, start):
-        s, L = self.s, self.w["layers"][i]
-        B, T, _ = x.shape
-        q = _rms(F.linear(x, L["wq"]), L["q_norm"], s.rms_eps)
-        k = _rms(F.linear(x, L["wk"]), L["k_norm"], s.rms_eps)
-        v = F.linear(x, L["wv"])
+    # ---- the PyTorch formulation of a forward pass (any device, any dtype)
+    def _heads(self, x, weight, norm, n_heads):
+        """One of the q / k / v projections of x [B, T, H] as heads [B, n_heads, T, head_dim]."""
+        s = self.s
+        y = F.linear(x, weight)
+        if norm is not None:
+            y = _rms(y, norm, s.rms_eps)
         if s.clip_qkv is not None:
-            q, k, v = q.clamp(-s.clip_qkv, s.clip_qkv), k.clamp(-s.clip_qkv, s.clip_qkv), v.clamp(-s.clip_qkv, s.clip_qkv)
-        q = q.view(B, T, s.heads, s.head_dim).transpose(1, 2)
-        k = k.view(B, T, s.kv_heads, s.head_dim).transpose(1, 2)
-        v = v.view(B, T, s.kv_heads, s.head_dim).transpose(1, 2)
-        cos, sin = self.cos[positions][:, None], self.sin[positions][:, None]
-        q, k = _rotate(q, cos, sin), _rotate(k, cos, sin)
-        if cache is not None:
-            cache.k[i, :, :, start:start + T] = k
-            cache.v[i, :, :, start:start + T] = v
-            k, v = cache.k[i, :, :, :start + T], cache.v[i, :, :, :start + T]
-        a = F.scaled_dot_product_attention(q, k, v, attn_mask=mask, enable_gqa=s.kv_heads != s.heads)
-        return F.linear(a.transpose(1, 2).reshape(B, T, s.heads * s.head_dim), L["wo"])
+            y = y.clamp(-s.clip_qkv, s.clip_qkv)
+        return y.unflatten(-1, (n_heads, s.head_dim)).transpose(1, 2)
 
-    def _prepare(self, tokens, cache, valid):
-        """Rotary positions and the attention mask of `tokens` [B, T] appended to `cache`."""
-        B, T = tokens.shape
-        dev = tokens.device
-        if valid is None:
-            valid = torch.ones(B, T, dtype=torch.bool, device=dev)
-        start = cache.filled if cache is not None else 0
-        base = cache.next_position if cache is not None else torch.zeros(B, dtype=torch.long, device=dev)
-        positions = (base[:, None] + valid.long().cumsum(1) - 1).clamp_(min=0)
+    def _attend(self, i, x, span, cache):
+        """Attention of layer i over the span's new positions (and what the cache already holds)."""
+        s, L = self.s, self.w["layers"][i]
+        cos, sin = self.cos[span.positions][:, None], self.sin[span.positions][:, None]
+        q = _rotate(self._heads(x, L["wq"], L["q_norm"], s.heads), cos, sin)
+        k = _rotate(self._heads(x, L["wk"], L["k_norm"], s.kv_heads), cos, sin)
+        v = self._heads(x, L["wv"], None, s.kv_heads)
         if cache is not None:
-            cache.real[:, start:start + T] = valid
-            keys_real = cache.real[:, :start + T]
-        else:
-            keys_real = valid
-        # query q (absolute index start+q) sees key j <= start+q that holds a real token; a padding
-        # query would see nothing, so it is allowed itself (its output is never used)
-        qi = torch.arange(start, start + T, device=dev)[:, None]
-        kj = torch.arange(start + T, device=dev)[None, :]
-        mask = (kj <= qi)[None] & keys_real[:, None, :]
-        mask = mask | ((kj == qi)[None] & ~mask.any(-1, keepdim=True))
-        return valid, start, base, positions, mask[:, None]  # the mask broadcasts over heads
+            new = slice(span.first, span.end)
+            cache.k[i, :, :, new], cache.v[i, :, :, new] = k, v
+            k, v = cache.k[i, :, :, :span.end], cache.v[i, :, :, :span.end]
+        a = F.scaled_dot_product_attention(q, k, v, attn_mask=span.visible, enable_gqa=s.kv_heads != s.heads)
+        return F.linear(a.transpose(1, 2).flatten(-2), L["wo"])
 
     @torch.no_grad()
     def forward(self, tokens, cache=None, valid=None):
@@ -202,16 +232,15 @@ class Decoder:
         padding). With a cache the tokens are appended after what it already holds."""
         s, W = self.s, self.w
         B, T = tokens.shape
-        valid, start, base, positions, mask = self._prepare(tokens, cache, valid)
+        span = Span(tokens, cache, valid)
         x = F.embedding(tokens, W["embed"])
         for i in range(s.layers):
             L = W["layers"][i]
-            x = x + self._attend(i, _rms(x, L["attn_norm"], s.rms_eps), positions, mask, cache, start)
+            x = x + self._attend(i, _rms(x, L["attn_norm"], s.rms_eps), span, cache)
             h = _rms(x, L["mlp_norm"], s.rms_eps).reshape(B * T, s.hidden)
             x = x + self.moe(i, h).view(B, T, s.hidden)
         if cache is not None:
-            cache.filled = start + T
-            cache.next_position = base + valid.long().sum(1)
+            span.commit(cache)
         return F.linear(_rms(x, W["final_norm"], s.rms_eps), W["lm_head"])
 
     @torch.no_grad()
@@ -226,10 +255,10 @@ class Decoder:
 
         s, W, E = self.s, self.w, kernels.ext()
         B, T = tokens.shape
-        valid, start, base, positions, mask = self._prepare(tokens, cache, valid)
+        span = Span(tokens, cache, valid)
         wqkv = self._stacked_qkv()
-        slot = torch.tensor([start], dtype=torch.long, device=tokens.device)
-        flat_positions = positions.reshape(-1).contiguous()
+        slot = torch.tensor([span.first], dtype=torch.long, device=tokens.device)
+        flat_positions = span.positions.reshape(-1).contiguous()
         x, xn = E.embed_rmsnorm(tokens.reshape(-1).contiguous(), W["embed"], W["layers"][0]["attn_norm"], s.rms_eps)
         for i in range(s.layers):
             L = W["layers"][i]
@@ -237,8 +266,8 @@ class Decoder:
             q = E.qk_norm_rope_cache(kernels.dense(xn, wqkv[i]), L["q_norm"], L["k_norm"], s.rms_eps, s.clip_qkv, self.cos,
                                      self.sin, flat_positions, slot, s.heads, s.kv_heads, s.head_dim, cache.k[i], cache.v[i])
             a = F.scaled_dot_product_attention(q.view(B, T, s.heads, s.head_dim).transpose(1, 2),
-                                               cache.k[i, :, :, :start + T], cache.v[i, :, :, :start + T], attn_mask=mask,
-                                               enable_gqa=s.kv_heads != s.heads)
+                                               cache.k[i, :, :, :span.end], cache.v[i, :, :, :span.end],
+                                               attn_mask=span.visible, enable_gqa=s.kv_heads != s.heads)
             o = kernels.dense(a.transpose(1, 2).reshape(B * T, s.heads * s.head_dim), L["wo"])
             x, h = E.add_rmsnorm(x, o, L["mlp_norm"], s.rms_eps, x_out=x)
             if self._own_moe and s.top_k <= 64:
@@ -247,8 +276,7 @@ class Decoder:
                 x, xn = E.combine_add_rmsnorm(y, pos_of, idx, x, after, s.rms_eps, x_out=x)
             else:
                 x, xn = E.add_rmsnorm(x, self.moe(i, h).contiguous(), after, s.rms_eps, x_out=x)
-        cache.filled = start + T
-        cache.next_position = base + valid.long().sum(1)
+        span.commit(cache)
         return kernels.dense(xn.view(B, T, s.hidden)[:, -1].contiguous(), W["lm_head"])
 
     def _prefill(self, tokens, cache, valid):
@@ -354,14 +382,9 @@ class Decoder:
         device synchronisations)."""
         import time
         dev, dtype = self.w["embed"].device, self.w["embed"].dtype
-        B, P = len(prompts), max(len(p) for p in prompts)
-        tokens = torch.zeros(B, P, dtype=torch.long)
-        valid = torch.zeros(B, P, dtype=torch.bool)
-        for b, p in enumerate(prompts):
-            tokens[b, P - len(p):] = torch.tensor(p, dtype=torch.long)
-            valid[b, P - len(p):] = True
+        tokens, valid = left_padded(prompts, dev)
+        B, P = tokens.shape
         cache = KVCache(self.s, B, P + max_new_tokens, dtype, dev)
-        tokens, valid = tokens.to(dev), valid.to(dev)
         if timings is not None:
             torch.cuda.synchronize()
             t0 = time.perf_counter()
@@ -423,13 +446,8 @@ class Decoder:
         tokens of each prompt (cut after `eos` if given). Without `eos` nothing is read back from
         the device until the end."""
         dev, dtype = self.w["embed"].device, self.w["embed"].dtype
-        B, P = len(prompts), max(len(p) for p in prompts)
-        tokens = torch.zeros(B, P, dtype=torch.long)
-        valid = torch.zeros(B, P, dtype=torch.bool)
-        for b, p in enumerate(prompts):
-            tokens[b, P - len(p):] = torch.tensor(p, dtype=torch.long)
-            valid[b, P - len(p):] = True
-        tokens, valid = tokens.to(dev), valid.to(dev)
+        tokens, valid = left_padded(prompts, dev)
+        B, P = tokens.shape
         cache = KVCache(self.s, B, P + max_new_tokens, dtype, dev)
         logits = self._prefill(tokens, cache, valid)
         first_logits = logits

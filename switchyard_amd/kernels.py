@@ -58,22 +58,38 @@ def pick(max_rows):
     return "gemm"
 
 
+# Above this many tokens "auto" never takes the weight-stream kernel: it handles 16 rows of an
+# expert per pass, a token picks an expert at most once, so up to 16 tokens one pass is certain
+# whatever the routing. Beyond that a popular expert takes a second pass and its many rows make
+# the stream compute-bound. Measured (us per experts() call, stream of calls; Zipf bias with
+# every token on the most popular expert): 17 tokens balanced 128 (gemv) / 135 (gemm), Zipf
+# 96 / 75; 24 tokens balanced 139 / 143, Zipf 125 / 87; 32 tokens balanced 147 / 146, Zipf
+# 160 / 111. Without a device read the routing is unknown, and what the MFMA tiles lose under
+# balanced routing (0 to 6 %) is small against what the stream loses under skew (20 to 30 %).
+GEMV_MAX_TOKENS = 16
+
+
 def _auto(n_tokens, n_choices, n_experts):
     """Mode for "auto" without a device read. No expert can have more rows than there are
-    tokens, so up to GEMV_MAX_ROWS tokens the answer is certain; above that the busiest expert
-    is estimated from the mean rows per expert (under near-uniform routing it sits about two
-    square roots of the mean above it). Both kernels are correct for any routing."""
+    tokens, so up to GEMV_MAX_ROWS tokens the answer is certain; up to GEMV_MAX_TOKENS the
+    busiest expert is estimated from the mean rows per expert (under near-uniform routing it
+    sits about two square roots of the mean above it); beyond, the MFMA tiles. Both kernels
+    are correct for any routing."""
     if n_tokens <= GEMV_MAX_ROWS:
         return "gemv"
+    if n_tokens > GEMV_MAX_TOKENS:
+        return "gemm"
     mean = n_choices / n_experts
     return pick(math.ceil(mean + 2.0 * math.sqrt(mean)))
 
 
 def ffn(x, a_rows, offsets, counts, wsorted, gate_up, down, rows, mode, host_counts=None):
-    """The experts over rows already sorted by expert: row i is x[a_rows[i]] (or x[i] when
-    a_rows is None); expert e owns rows offsets[e]:offsets[e+1]. Returns each row's expert
-    output scaled by its router weight, [rows, H]. `counts` and `host_counts` are accepted
-    for the reference's call shape; nothing here waits for the GPU."""
+    """Both projections of the experts for `rows` sorted rows -> y [rows, H], router weight
+    already applied. offsets [E + 1] cuts the sorted rows into one run per expert; sorted row i
+    reads x[a_rows[i]] (x[i] if a_rows is None), so the unsorted activations are never copied.
+    mode is "gemv" or "gemm" ("cublas" means "gemm" here). `counts` and `host_counts` only keep
+    the reference's argument list (kernels.py:48): no launch here depends on a value read
+    back from the GPU."""
     E = ext()
     if rows == 0:
         return torch.empty(0, down.shape[1], dtype=x.dtype, device=x.device)
@@ -89,10 +105,11 @@ def ffn(x, a_rows, offsets, counts, wsorted, gate_up, down, rows, mode, host_cou
 
 
 def experts(h, idx, w, gate_up, down, mode="auto"):
-    """The experts of one MoE layer on this GPU, for routing (idx, w) computed already:
-    sort by expert, SwiGLU projection reading rows of h in place, down projection scaled by
-    the router weights, combine. idx int32 [N, k] in 0..E-1 local expert ids.
-    mode: "gemv" (streams weights; few rows per expert), "gemm" (MFMA tiles), or "auto"."""
+    """Everything of the layer after routing: h [N, H], idx int32 [N, k] (expert ids
+    0..E-1), w [N, k] -> out [N, H] = sum over each token's k choices of
+    w * expert(h[token]). Four launches and no host read: counting sort, gate/up projection with
+    SwiGLU, down projection times w, fp32 combine in expert order. "auto" picks the weight-stream
+    kernel or the MFMA tiles from the token count (see _auto); "gemv" / "gemm" force one."""
     E = ext()
     N = h.shape[0]
     idx = idx.contiguous()

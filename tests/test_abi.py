@@ -153,3 +153,41 @@ def test_bench_refuses_more_than_one_gpu_and_needs_a_gpu():
     if not torch.cuda.is_available():
         one = subprocess.run([sys.executable, bench], capture_output=True, text=True, timeout=120)
         assert one.returncode != 0 and "no GPU" in one.stderr
+
+
+def test_the_reference_module_path_serves_the_same_names_and_signatures():
+    """`from switchyard import kernels` is the reference's import (switchyard/kernels.py:12-93);
+    the parameters and defaults below are the reference's, and `ext()` offers the five methods of
+    its native module that the one-GPU path uses (moe_kernels.cu:491-495) with their arguments
+    (:73, :142, :264-266, :385-386, :435)."""
+    import inspect
+
+    from switchyard import kernels as drop_in
+
+    assert drop_in.moe_layer is kernels.moe_layer and drop_in.ext is kernels.ext
+    want = {
+        "ext": [],
+        "tile_offsets": ["counts", ("block", 64)],
+        "route": ["h", "router", "top_k", "norm_topk_prob"],
+        "pick": ["max_rows"],
+        "ffn": ["x", "a_rows", "offsets", "counts", "wsorted", "gate_up", "down", "rows", "mode", ("host_counts", None)],
+        "experts": ["h", "idx", "w", "gate_up", "down", ("mode", "auto")],
+        "moe_layer": ["h", "router", "gate_up", "down", "top_k", "norm_topk_prob", ("mode", "auto")],
+    }
+    for name, params in want.items():
+        sig = inspect.signature(getattr(drop_in, name))
+        got = [(p.name, p.default) if p.default is not inspect.Parameter.empty else p.name for p in sig.parameters.values()]
+        assert got == params, name
+    assert isinstance(drop_in.GEMV_MAX_ROWS, int) and isinstance(drop_in.GEMM_MAX_ROWS, int)
+    assert sorted(drop_in.__all__) == sorted(list(want) + ["GEMV_MAX_ROWS", "GEMM_MAX_ROWS"])
+    native = {
+        "route": ["logits", "k", "norm"],
+        "sort_by_expert": ["idx", "w", "E"],
+        "grouped_gemm": ["A", "a_rows", "B", "offsets", "tile_offsets", "total_tiles", "rows", "swiglu", "scale"],
+        "grouped_gemv": ["A", "a_rows", "B", "offsets", "rows", "swiglu", "scale"],
+        "combine": ["y", "pos_of", "idx", "n_tokens"],
+    }
+    for name, params in native.items():
+        sig = inspect.signature(getattr(_abi.Ext, name))
+        required = [p.name for p in sig.parameters.values() if p.name != "self" and p.default is inspect.Parameter.empty]
+        assert required == params, name

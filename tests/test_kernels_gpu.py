@@ -337,7 +337,7 @@ def test_olmoe_layer_decode_and_prefill(K, olmoe, N, mode):
         assert err <= max(2 * err_half, 2e-3), (err, err_half)
 
 
-@pytest.mark.parametrize("N", [64, 1024])
+@pytest.mark.parametrize("N", [17, 24, 32, 64, 1024])   # 17-32: "auto" decides from the mean and may meet > 16 rows in an expert
 @pytest.mark.parametrize("kind", ["zipf", "adversarial"])
 def test_skewed_routing_is_exact_and_deterministic(K, olmoe, N, kind):
     router, gu, dn = olmoe
@@ -349,7 +349,7 @@ def test_skewed_routing_is_exact_and_deterministic(K, olmoe, N, kind):
     if kind == "adversarial":
         assert counts.tolist() == [N] * 8 + [0] * 56
     else:
-        assert counts.max().item() >= 3 * counts.float().mean().item()
+        assert counts.max().item() >= (3 if N >= 64 else 2.5) * counts.float().mean().item()
     half = O.experts_loop(h, idx.long(), w, gu, dn)
     for mode in ("gemv", "gemm", "auto"):
         a = K.experts(h, idx, w, gu, dn, mode)
