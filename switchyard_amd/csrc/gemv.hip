@@ -23,7 +23,7 @@
 // Rows. The expert's rows (up to `row_cap` <= 16 per pass, in quads of 4) are staged in LDS,
 // padded so that the 128-bit operand reads are bank-conflict free, and shared by the
 // workgroup's 4 wavefronts, which split the units of the current expert between them and
-// otherwise run independently. Loads are issued one chunk (4 steps) ahead of the MFMAs that
+// otherwise run independently. Loads are issued one chunk (4 or 8 steps) ahead of the MFMAs that
 // consume them, through a buffer descriptor whose range check masks ragged edges without
 // branches. An expert with more rows than `row_cap` takes further passes over its weights.
 //
@@ -39,7 +39,7 @@ constexpr int UNIT_COLS = 4;    // output columns per unit (MFMA M)
 constexpr int QUAD = 4;         // rows of the expert per MFMA (MFMA N)
 constexpr int MAX_QUADS = 4;    // up to 16 rows per pass
 constexpr int STEP_K = 128;     // K covered by one load instruction (16 blocks x 8 halves)
-constexpr int CH = 4;           // load steps per chunk
+constexpr int CH_SHORT = 4, CH_LONG = 8;  // load steps per chunk (a template parameter: see launch_gemv)
 constexpr int ROW_PAD = 32;     // halves of padding per staged row (64 bytes)
 constexpr int MAX_E = 1024;     // experts whose ids fit the LDS list
 
@@ -62,6 +62,7 @@ __device__ __forceinline__ float sum_blocks(float v) {
   return v;
 }
 
+template <int CH>
 struct Chunk {
   half8_t w[CH];
 };
@@ -76,7 +77,7 @@ struct Pass {
 
 // One wavefront streams units [unit0, unit0 + nunits) of one expert against NQ staged quads.
 // EXACT: K is a multiple of a chunk (512) and Nout of a unit (4), so nothing needs masking.
-template <bool SWIGLU, bool SCALE, bool EXACT, int NQ>
+template <bool SWIGLU, bool SCALE, bool EXACT, int CH, int NQ>
 __device__ __forceinline__ void run_pass(const Pass& p) {
   const int lane = threadIdx.x & 63, blk = lane >> 2, sub = lane & 3;
   const int klane = blk * 8;
@@ -92,7 +93,7 @@ __device__ __forceinline__ void run_pass(const Pass& p) {
   // ---- issue side: part `ipt` of unit `iun`, chunk `ich` (counted from the unit's start `irot`)
   // is the next to load
   int iun = 0, ipt = 0, ich = 0, irot = rot0;
-  auto issue = [&](Chunk& c) {
+  auto issue = [&](Chunk<CH>& c) {
     const int col = (p.unit0 + iun) * UNIT_COLS + sub;
     const int wr = ipt ? p.Nout + col : col;
     unsigned lane_off = ((unsigned)wr * (unsigned)p.K + (unsigned)klane) * 2u;
@@ -122,7 +123,7 @@ __device__ __forceinline__ void run_pass(const Pass& p) {
   for (int q = 0; q < NQ; ++q) acc[q] = gate[q] = float4_t{0.f, 0.f, 0.f, 0.f};
   const half_t* xlane = p.xs + sub * p.RS + klane;  // row `sub` of quad 0 at this lane's K offset
 
-  auto compute = [&](const Chunk& c) {
+  auto compute = [&](const Chunk<CH>& c) {
 #pragma unroll
     for (int s = 0; s < CH; ++s) {
       const int at = cch * CH + s + crot;
@@ -180,7 +181,7 @@ __device__ __forceinline__ void run_pass(const Pass& p) {
   // chunk q+1 is in flight while chunk q is multiplied
   const int total = p.nunits * PARTS * p.nchunks;
   if (total <= 0) return;
-  Chunk c0, c1;
+  Chunk<CH> c0, c1;
   issue(c0);
   int q = 0;
   for (; q + 3 <= total; q += 2) {
@@ -198,7 +199,7 @@ __device__ __forceinline__ void run_pass(const Pass& p) {
   }
 }
 
-template <bool SWIGLU, bool SCALE, bool EXACT>
+template <bool SWIGLU, bool SCALE, bool EXACT, int CH>
 __global__ void __launch_bounds__(GEMV_THREADS)
 gemv_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const half_t* __restrict__ B,
             const int* __restrict__ offsets, int E, int Nout, int K, const half_t* __restrict__ scale,
@@ -267,10 +268,10 @@ gemv_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const 
       p.r0 = r0;
       p.nr = nr;
       switch (nq) {
-        case 1: run_pass<SWIGLU, SCALE, EXACT, 1>(p); break;
-        case 2: run_pass<SWIGLU, SCALE, EXACT, 2>(p); break;
-        case 3: run_pass<SWIGLU, SCALE, EXACT, 3>(p); break;
-        default: run_pass<SWIGLU, SCALE, EXACT, 4>(p); break;
+        case 1: run_pass<SWIGLU, SCALE, EXACT, CH, 1>(p); break;
+        case 2: run_pass<SWIGLU, SCALE, EXACT, CH, 2>(p); break;
+        case 3: run_pass<SWIGLU, SCALE, EXACT, CH, 3>(p); break;
+        default: run_pass<SWIGLU, SCALE, EXACT, CH, 4>(p); break;
       }
     }
     at += count;
@@ -285,7 +286,11 @@ int launch_gemv(const void* A, const int32_t* a_rows, const void* B, const int32
   int row_cap = (bound + QUAD - 1) / QUAD * QUAD;
   row_cap = row_cap > MAX_QUADS * QUAD ? MAX_QUADS * QUAD : row_cap;
   const size_t lds = (size_t)row_cap * (K + ROW_PAD) * sizeof(half_t) + (size_t)(E + 1) * sizeof(int);
-  const bool exact = K % (CH * STEP_K) == 0 && Nout % UNIT_COLS == 0;
+  // Loads in flight per wavefront: a chunk of 4 KB, or of 8 KB where a unit is long enough to be
+  // cut into such chunks (gate and up rows of 2048 at 8 tokens: 56.6 us against 57.5; for rows of
+  // 1024 the longer chunk is one per unit and loses: 34.8 us against 30.6).
+  const bool long_chunks = swiglu && K % (CH_LONG * STEP_K) == 0 && K >= 2 * CH_LONG * STEP_K;
+  const bool exact = K % (CH_SHORT * STEP_K) == 0 && Nout % UNIT_COLS == 0;
   // persistent: a fixed number of workgroups per CU, but no more than there are units. Two per
   // CU stream best when a unit is 32 KB of weights (gate and up rows of 2048: 57.8 us against
   // 59.0 and 63.4 with three and four), four when it is 8 KB (rows of 1024: 31.8 us against
@@ -303,9 +308,10 @@ int launch_gemv(const void* A, const int32_t* a_rows, const void* B, const int32
   const half_t* s = (const half_t*)scale;
   half_t* c = (half_t*)C;
   void (*kern)(const half_t*, const int*, const half_t*, const int*, int, int, int, const half_t*, half_t*, int);
-  if (swiglu) kern = exact ? gemv_kernel<true, false, true> : gemv_kernel<true, false, false>;
-  else if (s) kern = exact ? gemv_kernel<false, true, true> : gemv_kernel<false, true, false>;
-  else kern = exact ? gemv_kernel<false, false, true> : gemv_kernel<false, false, false>;
+  if (swiglu && long_chunks && exact) kern = gemv_kernel<true, false, true, CH_LONG>;
+  else if (swiglu) kern = exact ? gemv_kernel<true, false, true, CH_SHORT> : gemv_kernel<true, false, false, CH_SHORT>;
+  else if (s) kern = exact ? gemv_kernel<false, true, true, CH_SHORT> : gemv_kernel<false, true, false, CH_SHORT>;
+  else kern = exact ? gemv_kernel<false, false, true, CH_SHORT> : gemv_kernel<false, false, false, CH_SHORT>;
   hipError_t attr = hipSuccess;
   if (lds > 48 * 1024) attr = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (attr != hipSuccess) return sy_fail(SY_ERR_LAUNCH, "grouped_gemv: cannot reserve %zu bytes of LDS", lds);
