@@ -383,6 +383,11 @@ def run_default(args):
     N = args.tokens
     cpu_layers = make_layers(args.layers)
     layers = [tuple(t.to(dev) for t in L) for L in cpu_layers]
+    if args.operands == "zeros":
+        # Same launches, same routing (the router keeps its values), expert weights all zero: the
+        # kernels run the same instructions on operands that toggle nothing, which separates what
+        # the schedule costs from what the chip's power management takes on random operands.
+        layers = [(r, torch.zeros_like(g), torch.zeros_like(d)) for r, g, d in layers]
     h_cpu = hidden(N)
     h = h_cpu.to(dev)
     mode = args.mode
@@ -427,7 +432,8 @@ def run_default(args):
         "data": "synthetic",
         "config": {"workload": f"olmoe_moe_layer_{'decode' if N <= 64 else 'prefill'}_{N}tok", "tokens": N,
                    "experts": E, "top_k": TOPK, "hidden": H, "expert_width": I, "mode": mode,
-                   "layers_rotated": n_layers, "experts_used_mean": used_mean, "spin_up_ms": SPIN_UP_MS},
+                   "layers_rotated": n_layers, "experts_used_mean": used_mean, "spin_up_ms": SPIN_UP_MS,
+                   **({"operands": "zero expert weights: NOT the benchmark"} if args.operands != "random" else {})},
         "timing": TIMING,
         "us_per_layer": ms_per_step * 1e3, "frac_of_hbm_peak": value / HBM_PEAK_GBS,
         "value_event_median": value_ev, "us_per_layer_event_median": ev_med * 1e3,
@@ -587,6 +593,8 @@ def main():
     ap.add_argument("--tokens", type=int, default=8)
     ap.add_argument("--mode", default="auto", choices=["auto", "gemv", "gemm"])
     ap.add_argument("--layers", type=int, default=4, help="distinct layers' weights to rotate through")
+    ap.add_argument("--operands", default="random", choices=["random", "zeros"],
+                    help='"zeros": expert weights of zero (a power experiment, with --no-cpu; not the benchmark)')
     ap.add_argument("--sweep", default=None, help='"all" or a comma list of token counts')
     ap.add_argument("--no-loops", action="store_true", help="sweep: skip the torch per-expert loops")
     ap.add_argument("--calibrate-copy", action="store_true",
