@@ -247,6 +247,11 @@ def test_grouped_gemv_with_many_experts(K, swiglu):
     ([1500, 2, 700], 192, 136),                     # many row tiles per expert, ragged columns
     ([(7 * i) % 23 for i in range(150)], 64, 40),         # 150 experts (several 64-lane scans), about 11 rows each
     ([((11 * i) % 7) * 90 for i in range(130)], 128, 264),   # 130 experts, 0 to 540 rows: the 256-row tile
+    # the 256-row tile as one stream per compute unit (four or more K slices, at most 128 experts):
+    ([300 + (i % 5) * 40 for i in range(100)], 256, 204),    # two experts per lane of the tile table; columns a multiple of 4 only
+    ([256] * 8, 256, 256),                                   # fewer tiles than workgroups, all of them full
+    ([5000, 3000, 1, 0, 257], 320, 201),                     # five slices, odd column count, 52 tiles of one expert
+    ([513, 576, 577, 129, 160, 161, 31, 32, 33, 700], 512, 136),   # every tile height from 1 to 8 blocks
 ])
 def test_grouped_gemm_every_tile_kind(K, counts, K_, Nout, swiglu):
     """Gathered rows, per-row scale (plain projection) or SwiGLU, experts with 0, 1 and many rows:
