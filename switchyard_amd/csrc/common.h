@@ -82,6 +82,18 @@ __device__ __forceinline__ half_t swiglu_f16(float gate, float up) {
   return (half_t)(s * u);
 }
 
+// The same for four outputs at a time: the roundings to fp16 pack two values per instruction, and
+// the last product is an fp16 multiply (the product of two fp16 numbers is exact in fp32, so it
+// rounds as the fp32 product rounded to fp16 does).
+__device__ __forceinline__ half4_t swiglu_f16x4(float4_t gate, float4_t up) {
+  const half4_t gh = __builtin_convertvector(gate, half4_t), uh = __builtin_convertvector(up, half4_t);
+  const float4_t g = __builtin_convertvector(gh, float4_t);
+  float4_t s;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) s[r] = g[r] * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(g[r] * -1.4426950408889634f));
+  return __builtin_convertvector(s, half4_t) * uh;
+}
+
 __device__ __forceinline__ uint64_t lanemask_lt() {
   return (1ull << (threadIdx.x & 63)) - 1ull;
 }

@@ -355,6 +355,46 @@ __device__ __forceinline__ void load_to_lds(int4_t rsrc, unsigned voffset, unsig
 }
 #pragma clang diagnostic pop
 
+typedef int int8v_t __attribute__((ext_vector_type(8)));
+
+// Four runs of 8 consecutive ints through the scalar cache, waited for here.
+__device__ __forceinline__ void scalar_load_4x8(const int* p0, const int* p1, const int* p2, const int* p3, int8v_t& a,
+                                                int8v_t& b, int8v_t& c, int8v_t& d) {
+  asm volatile(
+      "s_load_dwordx8 %0, %4, 0x0\n\t"
+      "s_load_dwordx8 %1, %5, 0x0\n\t"
+      "s_load_dwordx8 %2, %6, 0x0\n\t"
+      "s_load_dwordx8 %3, %7, 0x0\n\t"
+      "s_waitcnt lgkmcnt(0)"
+      : "=&s"(a), "=&s"(b), "=&s"(c), "=&s"(d)
+      : "s"(p0), "s"(p1), "s"(p2), "s"(p3));
+}
+
+typedef int int16v_t __attribute__((ext_vector_type(16)));
+// scale[first + l] for l = 0..31 (first is the same in the whole wavefront): 17 dwords from the
+// dword at or below scale + first through the scalar cache, waited for here; a lane picks its
+// half. The run is moved up where it would pass the end of the M scales (M >= 34); lanes whose
+// row is past the end get whatever is there.
+__device__ __forceinline__ half_t scale_of_row(const half_t* scale, int M, int first, int l) {
+  const uint64_t want = (uint64_t)(scale + first), end = ((uint64_t)(scale + M) + 3) & ~(uint64_t)3;
+  uint64_t from = want & ~(uint64_t)3;
+  from = from < end - 68 ? from : end - 68;
+  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)from), hi = __builtin_amdgcn_readfirstlane((unsigned)(from >> 32));
+  from = ((uint64_t)hi << 32) | lo;
+  int16v_t words;
+  int word;
+  asm volatile(
+      "s_load_dwordx16 %0, %2, 0x0\n\t"
+      "s_load_dword %1, %2, 0x40\n\t"
+      "s_waitcnt lgkmcnt(0)"
+      : "=&s"(words), "=&s"(word)
+      : "s"((const unsigned*)from));
+  const int h = (int)((want - from) >> 1) + l;
+#pragma unroll
+  for (int d = 0; d < 16; ++d) word = (h >> 1) == d ? words[d] : word;
+  return __builtin_bit_cast(half_t, (unsigned short)((h & 1) ? (unsigned)word >> 16 : (unsigned)word));
+}
+
 template <int EPL>
 struct ExpertTable {
   int first[EPL], count[EPL], tiles[EPL], lo[EPL];  // lane x holds experts x, x + 64, ...
@@ -465,6 +505,24 @@ gemm_stream_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows,
     t.b_hi = (unsigned)(be >> 32) & 0xffffu;
     t.rot = K % 2048 == 0 ? (e * 5) % nk : 0;
     const int nrows = t.row_end - t.row0;
+    // Row numbers come through the scalar path (its own counter: the vector loads in flight are
+    // counted by hand and must not be waited for here), the 8 rows of a load in one request and
+    // the tile's four requests in flight together. At the very end of the list the 8 are taken
+    // from further up and a lane picks its own from there.
+    int8v_t numbers[LOADS];
+    int mine[LOADS];
+    if (a_rows) {
+      static_assert(LOADS == 4, "one request per load of the tile");
+      const int* from[LOADS];
+#pragma unroll
+      for (int q = 0; q < LOADS; ++q) {
+        const int want = t.row0 + 8 * (WAVES * q + wave);
+        const int first = __builtin_amdgcn_readfirstlane(max(0, min(want, M - 8)));
+        from[q] = a_rows + first;
+        mine[q] = (lane >> 3) + (want - first);
+      }
+      scalar_load_4x8(from[0], from[1], from[2], from[3], numbers[0], numbers[1], numbers[2], numbers[3]);
+    }
 #pragma unroll
     for (int q = 0; q < LOADS; ++q) {
       const int rbase = 8 * (WAVES * q + wave);     // the 8 rows this load brings
@@ -472,14 +530,9 @@ gemm_stream_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows,
       const unsigned chunk = (unsigned)((lane & 7) ^ ((r >> 1) & 7));
       int src = t.row0 + r;
       if (a_rows) {
-        // row numbers through the scalar path (its own counter: the vector loads in flight are
-        // counted by hand and must not be waited for here)
         int picked = 0;
 #pragma unroll
-        for (int jj = 0; jj < 8; ++jj) {
-          const int v = a_rows[__builtin_amdgcn_readfirstlane(min(t.row0 + rbase + jj, M - 1))];
-          picked = (lane >> 3) == jj ? v : picked;
-        }
+        for (int jj = 0; jj < 8; ++jj) picked = mine[q] == jj ? numbers[q][jj] : picked;
         src = picked;
       }
       oa[q] = r < nrows ? ((unsigned)src * (unsigned)K + chunk * 8u) * 2u : OUT_OF_RANGE;
@@ -652,85 +705,89 @@ gemm_stream_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows,
       const int last_stage = b_stage == 0 ? BIG_B_STAGES - 1 : b_stage - 1;   // b_stage already points at the next tile's slice 0
       char* turn = lds + BIG_A_STAGES * BIG_A_BYTES + last_stage * BIG_B_BYTES + wave * 1024;   // piece c at + c * 8 KB
       const int hsel = lane >> 5;
+      // the tile's columns all exist and rows of C are 16-byte aligned: no column is checked
+      auto blocks = [&](auto whole_columns) {
+        constexpr bool WHOLE = decltype(whole_columns)::value;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int rblock = cur.row0 + (2 * i + wm) * 32;
-        if (rblock >= cur.row_end) continue;   // the same for the whole wavefront
-        const float sc_row = SCALE && rblock + l32 < cur.row_end ? (float)scale[rblock + l32] : 1.f;
-        // lane (l32, hsel) holds row l32 of the block, columns 32 j + 8 q + 4 hsel + 0..3
-        char* wrow = turn + (l32 >> 3) * 8192 + (l32 & 7) * 128;
-        const int wkey = (l32 >> 1) & 15;
+        for (int i = 0; i < 4; ++i) {
+          const int rblock = cur.row0 + (2 * i + wm) * 32;
+          if (rblock >= cur.row_end) continue;   // the same for the whole wavefront
+          // the block's 32 scales come through the scalar cache: a vector load here would have to be
+          // waited for, and with it every load of the stream that is in flight and every store so far
+          const half_t sc = SCALE ? scale_of_row(scale, M, rblock, l32) : (half_t)1.f;
+          const half4_t sc4 = {sc, sc, sc, sc};
+          // lane (l32, hsel) holds row l32 of the block, columns 32 j + 8 q + 4 hsel + 0..3
+          char* wrow = turn + (l32 >> 3) * 8192 + (l32 & 7) * 128;
+          const int wkey = (l32 >> 1) & 15;
 #pragma unroll
-        for (int j = 0; j < NB; ++j)
+          for (int j = 0; j < NB; ++j)
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            half4_t o;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              const float v = acc[i][j][4 * q + r];
-              o[r] = SCALE ? (half_t)((float)(half_t)v * sc_row) : (half_t)v;
+            for (int q = 0; q < 4; ++q) {
+              const float4_t v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+              half4_t o = __builtin_convertvector(v, half4_t);   // two packed conversions
+              // the product of two fp16 numbers is exact in fp32, so the fp16 multiply rounds as
+              // (half)((float)o * (float)scale) does
+              if (SCALE) o = o * sc4;
+              *reinterpret_cast<half4_t*>(wrow + (((8 * j + 2 * q + hsel) ^ wkey) * 8)) = o;
             }
-            *reinterpret_cast<half4_t*>(wrow + (((8 * j + 2 * q + hsel) ^ wkey) * 8)) = o;
-          }
-        // piece t holds rows 8 t .. 8 t + 7 of the block; lane = 8 * row + 16-byte part
-        const int rr = lane >> 3, part = lane & 7;
+          // piece t holds rows 8 t .. 8 t + 7 of the block; lane = 8 * row + 16-byte part
+          const int rr = lane >> 3, part = lane & 7;
+          const int c0 = cur.n0 + wn * (NB * 32) + 8 * part;
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const int brow = 8 * t + rr, rkey = (brow >> 1) & 15;
-          half8_t v = *reinterpret_cast<const half8_t*>(turn + t * 8192 + rr * 128 + ((part ^ (rkey >> 1)) * 16));
-          if (rkey & 1) v = __builtin_shufflevector(v, v, 4, 5, 6, 7, 0, 1, 2, 3);   // the XOR swapped the part's two slots
-          const int row = rblock + brow, c0 = cur.n0 + wn * (NB * 32) + 8 * part;
-          if (row < cur.row_end) {
-            half_t* dst = C + (size_t)row * Nout + c0;
-            if (c0 + 7 < Nout && (Nout & 7) == 0) {
-              *reinterpret_cast<half8_t*>(dst) = v;
-            } else {
+          for (int t = 0; t < 4; ++t) {
+            const int brow = 8 * t + rr, rkey = (brow >> 1) & 15;
+            half8_t v = *reinterpret_cast<const half8_t*>(turn + t * 8192 + rr * 128 + ((part ^ (rkey >> 1)) * 16));
+            if (rkey & 1) v = __builtin_shufflevector(v, v, 4, 5, 6, 7, 0, 1, 2, 3);   // the XOR swapped the part's two slots
+            const int row = rblock + brow;
+            if (row < cur.row_end) {
+              half_t* dst = C + (size_t)row * Nout + c0;
+              if (WHOLE) {
+                *reinterpret_cast<half8_t*>(dst) = v;
+              } else {
 #pragma unroll
-              for (int r = 0; r < 8; ++r)
-                if (c0 + r < Nout) dst[r] = v[r];
+                for (int r = 0; r < 8; ++r)
+                  if (c0 + r < Nout) dst[r] = v[r];
+              }
             }
           }
         }
-      }
+      };
+      if ((Nout & 7) == 0 && cur.n0 + COLS <= Nout) blocks(std::true_type{});
+      else blocks(std::false_type{});
       // the buffer is the stream's again: every read of it has returned before its loads go out
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
       for (int q = 0; q < LOADS; ++q) issue_weights(nk + 2, last_stage, q);
     } else {
-    // ---- epilogue, 8 bytes of a row per lane (with SwiGLU: turning the outputs round and holding the
-    // prefetch back, as above, costs the gate/up projection 3 %: 296 us against 287)
-    const int chalf = (lane >> 5) * 4;
+      // ---- epilogue with SwiGLU, 8 bytes of a row per lane (turning the outputs round and holding
+      // the prefetch back, as above, costs the gate/up projection 3 %: 296 us against 287)
+      static_assert(NB == 2, "a wavefront holds gate and up of the same 32 columns");
+      const int chalf = (lane >> 5) * 4;
+      auto blocks = [&](auto whole_columns) {
+        constexpr bool WHOLE = decltype(whole_columns)::value;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int row = cur.row0 + (2 * i + wm) * 32 + l32;
-      if (row >= cur.row_end) continue;
-      const float sc_row = SCALE ? (float)scale[row] : 1.f;
-      half_t* crow = C + (size_t)row * Nout;
-      constexpr int NJ = SWIGLU ? NB / 2 : NB;
+        for (int i = 0; i < 4; ++i) {
+          const int row = cur.row0 + (2 * i + wm) * 32 + l32;
+          if (row >= cur.row_end) continue;
+          half_t* crow = C + (size_t)row * Nout + cur.n0 + wn * 32 + chalf;
 #pragma unroll
-      for (int j = 0; j < NJ; ++j) {
-        const int cbase = cur.n0 + wn * (NJ * 32) + j * 32 + chalf;
+          for (int q = 0; q < 4; ++q) {
+            const float4_t g = {acc[i][0][4 * q], acc[i][0][4 * q + 1], acc[i][0][4 * q + 2], acc[i][0][4 * q + 3]};
+            const float4_t u = {acc[i][1][4 * q], acc[i][1][4 * q + 1], acc[i][1][4 * q + 2], acc[i][1][4 * q + 3]};
+            const half4_t o = swiglu_f16x4(g, u);
+            if (WHOLE) {
+              *reinterpret_cast<half4_t*>(crow + 8 * q) = o;
+            } else {
+              const int c0 = cur.n0 + wn * 32 + chalf + 8 * q;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int c0 = cbase + 8 * q;
-          half4_t o;
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const float v = acc[i][j][4 * q + r];
-            if (SWIGLU) o[r] = swiglu_f16(v, acc[i][SWIGLU ? j + NB / 2 : j][4 * q + r]);
-            else if (SCALE) o[r] = (half_t)((float)(half_t)v * sc_row);
-            else o[r] = (half_t)v;
-          }
-          if (c0 + 3 < Nout && (Nout & 3) == 0) {
-            *reinterpret_cast<half4_t*>(crow + c0) = o;
-          } else {
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-              if (c0 + r < Nout) crow[c0 + r] = o[r];
+              for (int r = 0; r < 4; ++r)
+                if (c0 + r < Nout) crow[8 * q + r] = o[r];
+            }
           }
         }
-      }
-    }
+      };
+      if ((Nout & 3) == 0 && cur.n0 + COLS <= Nout) blocks(std::true_type{});
+      else blocks(std::false_type{});
     }
     if (!nxt.valid) break;
     cur = nxt;
