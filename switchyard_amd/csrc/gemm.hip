@@ -601,7 +601,8 @@ gemm_stream_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows,
   const char* as = lds + (wm * 32 + l32) * BIG_ROW_BYTES;
   const char* bs = lds + BIG_A_STAGES * BIG_A_BYTES + l32 * BIG_ROW_BYTES;
 
-  // ---- fill the pipe for the first tile: rows 0, weights 0 | rows 1, weights 1 | weights 2
+  // ---- fill the pipe for the first tile: rows 0, weights 0 | rows 1, weights 1 (the first
+  // iteration asks for weights 2)
 #pragma unroll
   for (int p = 0; p < 2; ++p) {
 #pragma unroll
@@ -609,11 +610,9 @@ gemm_stream_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows,
 #pragma unroll
     for (int q = 0; q < LOADS; ++q) issue_weights(p, p, q);
   }
-#pragma unroll
-  for (int q = 0; q < LOADS; ++q) issue_weights(2, 2, q);
   // the second tile is looked up while the first tile's loads are on their way
   lookup(logical_of(round++), nxt, oa_n, ob_n);
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * LOADS) : "memory");
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * LOADS) : "memory");
   __syncthreads();
   int a_stage = 0, b_stage = 0;  // where the current tile's slice 0 is
 
@@ -644,16 +643,18 @@ gemm_stream_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows,
       for (int r = 0; r < READS; ++r) read(a_stage * BIG_A_BYTES, b_stage * BIG_B_BYTES, 0, r);
       for (int kt = 0; kt < nk; ++kt) {
         const int a_next = a_stage ^ 1, b_next = b_stage == BIG_B_STAGES - 1 ? 0 : b_stage + 1;
+        const int b_free = b_stage == 0 ? BIG_B_STAGES - 1 : b_stage - 1;   // the buffer slice kt - 1 has left
         const int sa = a_stage * BIG_A_BYTES, sb = b_stage * BIG_B_BYTES;
+        // A compute unit takes a load of this kind every 25 to 40 cycles, and a wavefront whose
+        // load is not taken issues no MFMA either: the eight loads of an iteration are spread over
+        // it, the weights (slice kt + 2) one or two after each of the first three steps, the rows
+        // after the barrier, instead of all 64 of the workgroup at once.
 #pragma unroll
         for (int s = 0; s < BIG_STEPS - 1; ++s) {
 #pragma unroll
           for (int r = 0; r < READS; ++r) read(sa, sb, s + 1, r);
 #pragma unroll
           for (int m = 0; m < MFMAS; ++m) mfma(s, m);
-        }
-#pragma unroll
-        for (int s = 0; s < BIG_STEPS - 1; ++s) {
 #pragma unroll
           for (int n = 0; n < PAIRS; ++n) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
@@ -661,21 +662,24 @@ gemm_stream_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows,
           }
           if (READS > PAIRS) __builtin_amdgcn_sched_group_barrier(0x100, READS - PAIRS, 0);
           if (MFMAS > PAIRS) __builtin_amdgcn_sched_group_barrier(0x008, MFMAS - PAIRS, 0);
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int q = 0; q < LOADS; ++q)
+            if (q * (BIG_STEPS - 1) / LOADS == s) issue_weights(kt + 2, b_free, q);
+          __builtin_amdgcn_sched_barrier(0);
         }
-        __builtin_amdgcn_sched_barrier(0);
         asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(LOADS) : "memory");
         __syncthreads();
 #pragma unroll
-        for (int part = 0; part < 2 * LOADS; ++part) {
+        for (int part = 0; part < LOADS; ++part) {
 #pragma unroll
           for (int r = 0; r < READS; ++r)
-            if (r * 2 * LOADS / (READS > 0 ? READS : 1) == part) read(a_next * BIG_A_BYTES, b_next * BIG_B_BYTES, 0, r);
+            if (r * LOADS / (READS > 0 ? READS : 1) == part) read(a_next * BIG_A_BYTES, b_next * BIG_B_BYTES, 0, r);
 #pragma unroll
           for (int m = 0; m < MFMAS; ++m)
-            if (m * 2 * LOADS / (MFMAS > 0 ? MFMAS : 1) == part) mfma(BIG_STEPS - 1, m);
+            if (m * LOADS / (MFMAS > 0 ? MFMAS : 1) == part) mfma(BIG_STEPS - 1, m);
           __builtin_amdgcn_sched_barrier(0);
-          if (part < LOADS) issue_rows(kt + 2, a_stage, part);
-          else if (!TURN || kt + 1 < nk) issue_weights(kt + 3, b_stage, part - LOADS);   // with TURN the tile's last one waits for the epilogue
+          issue_rows(kt + 2, a_stage, part);
           __builtin_amdgcn_sched_barrier(0);
         }
         a_stage = a_next;
@@ -754,10 +758,9 @@ gemm_stream_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows,
       };
       if ((Nout & 7) == 0 && cur.n0 + COLS <= Nout) blocks(std::true_type{});
       else blocks(std::false_type{});
-      // the buffer is the stream's again: every read of it has returned before its loads go out
+      // the buffer is the stream's again (the next tile's first iteration fills it): every read
+      // of it has returned by then
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-#pragma unroll
-      for (int q = 0; q < LOADS; ++q) issue_weights(nk + 2, last_stage, q);
     } else {
       // ---- epilogue with SwiGLU, 8 bytes of a row per lane (turning the outputs round and holding
       // the prefetch back, as above, costs the gate/up projection 3 %: 296 us against 287)
