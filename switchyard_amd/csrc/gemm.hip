@@ -610,8 +610,6 @@ gemm_stream_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows,
 #pragma unroll
     for (int q = 0; q < LOADS; ++q) issue_weights(p, p, q);
   }
-  // the second tile is looked up while the first tile's loads are on their way
-  lookup(logical_of(round++), nxt, oa_n, ob_n);
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * LOADS) : "memory");
   __syncthreads();
   int a_stage = 0, b_stage = 0;  // where the current tile's slice 0 is
@@ -684,6 +682,9 @@ gemm_stream_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows,
         }
         a_stage = a_next;
         b_stage = b_next;
+        // The tile after this one is looked up here, where the MFMAs of the other wavefront of the
+        // SIMD cover it; its offsets are first needed two iterations before this tile ends.
+        if (kt == 0) lookup(logical_of(round++), nxt, oa_n, ob_n);
       }
     };
     const int nrows = cur.row_end - cur.row0;
@@ -799,7 +800,6 @@ gemm_stream_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows,
       oa_c[q] = oa_n[q];
       ob_c[q] = ob_n[q];
     }
-    lookup(logical_of(round++), nxt, oa_n, ob_n);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no load may land in LDS after this workgroup has given it back
 }
