@@ -747,7 +747,9 @@ gemm_stream_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows,
             if (row < cur.row_end) {
               half_t* dst = C + (size_t)row * Nout + c0;
               if (WHOLE) {
-                *reinterpret_cast<half8_t*>(dst) = v;
+                // whole lines that nothing reads again before the launch ends: written through, so
+                // that the caches have less to write back when it does
+                __builtin_nontemporal_store(v, reinterpret_cast<half8_t*>(dst));
               } else {
 #pragma unroll
                 for (int r = 0; r < 8; ++r)
