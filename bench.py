@@ -257,6 +257,35 @@ def projection_rooflines(kernels, N, layers, mode, reps, warmup):
     return out[0], out[1]
 
 
+def library_batched_gemm(layers, N, reps=50):
+    """What the vendor library's batched GEMM takes for the two projections of N tokens under
+    perfectly even routing: torch.bmm over E problems of N*k/E rows each, every expert with its
+    own weights of a rotated layer (so they stream from HBM as in the real launch), random fp16
+    operands. No gather, no SwiGLU, no routing weights, no ragged experts: the same flops as
+    `prefill.roofline` counts, on the easiest terms, as a measure of what this GPU sustains on
+    this shape."""
+    dev = layers[0][1].device
+    n = N * TOPK // E
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(E, n, H, generator=g).half().to(dev)
+    a = torch.randn(E, n, I, generator=g).mul_(0.3).half().to(dev)
+    out = {"rows_per_expert": n, "what": "torch.bmm, E problems, each expert's own weights, no gather/SwiGLU/scale"}
+    for name, lhs, pick, flops in (("gate_up", x, 1, 4.0), ("down", a, 2, 2.0)):
+        calls = [0]
+
+        def fn():
+            w = layers[calls[0] % len(layers)][pick]
+            calls[0] += 1
+            return torch.bmm(lhs, w.transpose(1, 2))
+
+        spin_up(fn, 20.0)
+        t = stream_times(fn, reps, 10)
+        ms = sum(t) / len(t)
+        out[name + "_us"] = ms * 1e3
+        out[name + "_frac_of_mfma_peak"] = E * n * flops * H * I / ms / 1e9 / MFMA_F16_PEAK_TFLOPS
+    return out
+
+
 def cpu_loop_baseline(h, router, gu, dn, used, reps=5):
     """The reference per-expert loop (switchyard/moe.py:34-42) restated in oracle/, fp32, on the host."""
     from oracle import moe_oracle as O
@@ -413,6 +442,10 @@ def run_default(args):
         big = max(PREFILL_SIZES)
         prefill = layer_record(kernels, big, layers, "gemm", 50, 5)
         prefill["roofline"], prefill["down_projection"] = projection_rooflines(kernels, big, layers, "gemm", 100, 5)
+        try:
+            prefill["library_batched_gemm_even_routing"] = library_batched_gemm(layers, big)
+        except Exception as exc:  # a comparison, not part of the metric
+            prefill["library_batched_gemm_even_routing"] = {"error": f"{type(exc).__name__}: {exc}"}
         prefill["other_sizes"] = {str(n): layer_record(kernels, n, layers, "gemm", 50, 5) for n in PREFILL_SIZES if n != big}
         gpu_loop = gpu_loop_baseline(layers)
         n_layers = len(layers)

@@ -279,6 +279,32 @@ def test_grouped_gemm_every_tile_kind(K, counts, K_, Nout, swiglu):
     assert torch.allclose(got, want, rtol=2.0 ** -9, atol=1e-2)
 
 
+def test_grouped_gemm_stream_tile_with_operands_at_odd_addresses(K):
+    """The 256-row tile reads row numbers and scales in runs through the scalar cache, from the
+    4-byte word at or below where they start and moved up where a run would pass the end: the
+    scales start 2 bytes and the row numbers 4 bytes into their allocations here, and the last
+    expert ends the list with a block of a single row."""
+    counts, K_, Nout = [300, 417, 1, 290, 513], 256, 256
+    E, rows = len(counts), sum(counts)
+    g = torch.Generator().manual_seed(5)
+    src = torch.randn(400, K_, generator=g).half()
+    a_rows = torch.randint(0, 400, (rows,), generator=g).int()
+    B = (torch.randn(E, Nout, K_, generator=g) * K_ ** -0.5).half()
+    scale = torch.rand(rows, generator=g).half()
+    offsets = torch.zeros(E + 1, dtype=torch.int32)
+    offsets[1:] = torch.cumsum(torch.tensor(counts), 0)
+    scale_dev = torch.cat([torch.zeros(1, dtype=torch.float16), scale]).to(DEV)[1:]
+    rows_dev = torch.cat([torch.zeros(1, dtype=torch.int32), a_rows]).to(DEV)[1:]
+    assert scale_dev.data_ptr() % 4 == 2 and rows_dev.data_ptr() % 8 == 4
+    got = K.ext().grouped_gemm(src.to(DEV), rows_dev, B.to(DEV), offsets.to(DEV), None, 0, rows, False, scale_dev).float().cpu()
+    A = src[a_rows.long()]
+    want = torch.empty(rows, Nout)
+    for e in range(E):
+        s, t = int(offsets[e]), int(offsets[e + 1])
+        want[s:t] = F.linear(A[s:t].float(), B[e].float()).half().float() * scale[s:t, None].float()
+    assert torch.allclose(got, want, rtol=2.0 ** -9, atol=1e-2)
+
+
 # ------------------------------------------------------------------ the layer, the reference's test
 @pytest.mark.parametrize("N", [1, 7, 64, 333, 2048])
 @pytest.mark.parametrize("skew", [0.0, 2.0])
