@@ -75,6 +75,14 @@ SY_API int sy_sort_by_expert_static(const int32_t* idx, const void* w, int w_byt
                                     int32_t* counts, int32_t* offsets, int32_t* token, void* wsorted,
                                     int32_t* pos_of, void* stream);
 
+/* The router GEMM and route() in ONE launch, for more tokens than a decode step has.
+ * Fuses F.linear(h, router) + route() (switchyard/kernels.py:30-32; kernel moe_kernels.cu:23-71):
+ * h f16 [N,H]; router f16 [E,H] -> logits f16 [N,E] (fp32 sums in a fixed order, rounded once),
+ * and from those logits exactly the outputs of sy_route (idx, w in f16).
+ * Limits: H a multiple of 512, E <= 128, k <= 8, N*H*2 < 2 GiB. N == 0 is a no-op. */
+SY_API int sy_router_route(const void* h, const void* router, int N, int H, int E, int k, int norm, void* logits,
+                           int32_t* idx, void* w, void* stream);
+
 /* Route and sort of a decode step in ONE launch (one workgroup).
  * Fuses route() (moe_kernels.cu:73-89) and sort_by_expert() (moe_kernels.cu:142-157), which the
  * reference's layer calls back to back (switchyard/kernels.py:91-93,84).
@@ -115,9 +123,10 @@ SY_API int sy_combine(const void* y, const int32_t* pos_of, const int32_t* idx, 
 
 /* Replaces moe_layer() (switchyard/kernels.py:91-93: route() with its router GEMM, :30-32, then
  * experts(), :76-88: sort -> pick -> ffn -> combine) in ONE call: the router's logits
- * (sy_router_logits, when `router` is given; with router NULL `logits` is an input), route and
- * sort (sy_route_sort when one_launch_front is nonzero, else sy_route and sy_sort_by_expert with
- * the given workspace), the gate/up projection (SwiGLU, rows of h gathered through `token`), the
+ * (when `router` is given: sy_router_logits up to 64 tokens, above that sy_router_route, which
+ * routes in the same launch and is also the first pass of the sort; with router NULL `logits` is
+ * an input), route and sort (sy_route_sort when one_launch_front is nonzero, else sy_route and
+ * sy_sort_by_expert with the given workspace), the gate/up projection (SwiGLU, rows of h gathered through `token`), the
  * down projection (x router weight) and sy_combine are enqueued back to back, exactly as the
  * separate calls would be.
  * h f16 [N,H]; router f16 [E,H] or NULL; logits f16 [N,E]; gate_up f16 [E,2I,H]; down f16

@@ -39,6 +39,8 @@ SIGNATURES = {
     "sy_moe_experts": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p,
                                 _c_int, _c_int, _c_int, _c_int] + [_c_void_p] * 11 + [_c_size_t, _c_void_p]),
     "sy_router_logits": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p]),
+    "sy_router_route": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p,
+                                 _c_void_p, _c_void_p]),
     "sy_add_rmsnorm": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_int, _c_int, _c_void_p, _c_void_p,
                                 _c_void_p]),
     "sy_embed_rmsnorm": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_float, _c_int, _c_int, _c_void_p, _c_void_p,
@@ -248,6 +250,27 @@ class Ext:
                    gate_up.data_ptr(), down.data_ptr(), H, I, int(bool(mfma_tiles)), int(bool(one_launch_front)),
                    *[base + s for s in starts[:9]], out.data_ptr(), base + starts[9] if need else None, need, _stream())
         return out
+
+    @staticmethod
+    def router_route_ok(N, H, E, k):
+        """Whether router_route (and moe_experts with a router, above 64 tokens) takes this shape."""
+        return N >= 1 and H >= 512 and H % 512 == 0 and E <= 128 and 1 <= k <= 8 and k <= E and N * H * 2 < 2 ** 31
+
+    def router_route(self, h, router, k, norm):
+        """h [N, H], router [E, H] -> (idx int32 [N, k], w f16 [N, k], logits f16 [N, E]): the
+        router GEMM and route in one launch (H a multiple of 512, at most 128 experts, top-8)."""
+        _check(h, "h", torch.float16)
+        _check(router, "router", torch.float16)
+        N, H = h.shape
+        E = router.shape[0]
+        if router.shape[1] != H:
+            raise RuntimeError("router_route: h and router must have the same width")
+        logits = torch.empty((N, E), dtype=torch.float16, device=h.device)
+        idx = torch.empty((N, int(k)), dtype=torch.int32, device=h.device)
+        w = torch.empty((N, int(k)), dtype=torch.float16, device=h.device)
+        self._call(self.lib.sy_router_route, h.data_ptr(), router.data_ptr(), N, H, E, int(k), int(bool(norm)),
+                   logits.data_ptr(), idx.data_ptr(), w.data_ptr(), _stream())
+        return idx, w, logits
 
     def router_logits(self, h, router):
         """h [N, H] @ router [E, H]^T -> logits [N, E] f16 by the library's own kernel (tens of rows)."""

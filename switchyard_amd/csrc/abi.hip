@@ -56,17 +56,29 @@ extern "C" SY_API int sy_moe_experts(const void* h, const void* router, void* lo
   // the projections address the gathered rows of h with 32-bit byte offsets
   SY_REQUIRE((long)N * H * 2 < (1l << 31), "moe_experts: h must stay under 2 GiB (%d rows of %d)", N, H);
   int rc;
-  if (router) {   // the router GEMM too: logits is then an output
-    rc = sy_router_logits(h, router, N, H, E, logits, stream);
+  if (router && N > 64) {
+    // beyond the decode kernels' range: one launch for the logits and route, which is also the
+    // sort's first pass where the sort runs over many workgroups
+    SY_REQUIRE(!one_launch_front, "moe_experts: one_launch_front with a router is for at most 64 tokens");
+    const bool counted = sy_router_route_counts(N, k) && sort_workspace && sort_workspace_bytes >= sy_sort_workspace_bytes(N, k, E);
+    rc = sy_router_route_counting(h, router, N, H, E, k, norm, logits, idx, w, counted ? sort_workspace : nullptr, stream);
     if (rc) return rc;
-  }
-  if (one_launch_front) {
-    rc = sy_route_sort(logits, N, E, k, norm, idx, w, counts, offsets, token, wsorted, pos_of, stream);
+    rc = counted ? sy_sort_assign_counted(idx, w, N, k, E, counts, offsets, token, wsorted, pos_of, sort_workspace, stream)
+                 : sy_sort_by_expert(idx, w, 2, N, k, E, counts, offsets, token, wsorted, pos_of, sort_workspace,
+                                     sort_workspace_bytes, stream);
   } else {
-    rc = sy_route(logits, SY_DTYPE_F16, N, E, k, norm, idx, w, stream);
-    if (rc) return rc;
-    rc = sy_sort_by_expert(idx, w, 2, N, k, E, counts, offsets, token, wsorted, pos_of, sort_workspace,
-                           sort_workspace_bytes, stream);
+    if (router) {   // the router GEMM too: logits is then an output
+      rc = sy_router_logits(h, router, N, H, E, logits, stream);
+      if (rc) return rc;
+    }
+    if (one_launch_front) {
+      rc = sy_route_sort(logits, N, E, k, norm, idx, w, counts, offsets, token, wsorted, pos_of, stream);
+    } else {
+      rc = sy_route(logits, SY_DTYPE_F16, N, E, k, norm, idx, w, stream);
+      if (rc) return rc;
+      rc = sy_sort_by_expert(idx, w, 2, N, k, E, counts, offsets, token, wsorted, pos_of, sort_workspace,
+                             sort_workspace_bytes, stream);
+    }
   }
   if (rc) return rc;
   const int M = N * k;

@@ -23,6 +23,14 @@ int sy_check_launch(const char* what);
 
 // Compute units of the current device (cached per device).
 int sy_compute_units();
+// sort.hip: the second launch of the sort over many workgroups, for a caller that has left the
+// per-piece histograms in the workspace itself (f16 weights, N*k above the one-workgroup limit)
+int sy_sort_assign_counted(const int32_t* idx, const void* w, int N, int k, int E, int32_t* counts, int32_t* offsets,
+                           int32_t* token, void* wsorted, int32_t* pos_of, void* workspace, void* stream);
+// front.hip: router logits + route in one launch; with `hist` also the sort's per-piece histograms
+int sy_router_route_counting(const void* h, const void* router, int N, int H, int E, int k, int norm, void* logits,
+                             int32_t* idx, void* w, void* hist, void* stream);
+bool sy_router_route_counts(int N, int k);
 
 #define SY_REQUIRE(cond, ...) \
   do {                        \

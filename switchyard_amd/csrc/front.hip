@@ -56,6 +56,158 @@ front_kernel(const half_t* __restrict__ logits, int N, int E, int k, int norm, i
                              reinterpret_cast<uint16_t*>(wsorted), pos_of, lds);
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// router_route: the router's logits, route and, when asked, the first pass of the sort, in one
+// launch, for more tokens than the decode path's kernels are for.
+//
+// At hundreds to thousands of tokens the library's GEMM for [N, H] x [E, H]^T (64 output
+// columns) takes about 14 us, the route launch 6 and the sort's counting launch 5, in front of
+// two projections; each is a launch's latency around very little work. Here a workgroup takes
+// 16 tokens: its wavefronts (16, or 4 where H is not a multiple of 2048 or there are more than
+// 64 experts) each multiply their share of H on v_mfma_f32_16x16x32_f16 (the tokens as the 16
+// rows, 16 experts per block as the columns, operands straight from memory: 16 bytes per lane,
+// 64 contiguous bytes of a row per instruction), the partial sums meet in LDS and are added in
+// a fixed order, rounded to f16 once (the logits, also written out), and the wavefronts then
+// route a token each from LDS with the code of route.hip. Everything here is latency, so the
+// workgroup is as wide as the shape allows: 21 us with 4 wavefronts at 4096 tokens. With `hist` the
+// workgroup is one piece of the sort (sort.hip): it owns piece / k tokens, 16 at a time, and
+// leaves the histogram of its choices where the sort's second launch expects it.
+//
+// Fuses F.linear(h, router) + route() of the reference (switchyard/kernels.py:30-32,
+// switchyard/csrc/moe_kernels.cu:23-89) and count_kernel (:91-104).
+constexpr int RR_TOKENS = 16, RR_KSTEP = 32;
+
+typedef float float4v_t __attribute__((ext_vector_type(4)));
+
+template <int PER_LANE, int RR_WAVES>
+__global__ void __launch_bounds__(RR_WAVES * WAVE)
+router_route_kernel(const half_t* __restrict__ h, const half_t* __restrict__ router, int N, int H, int E, int k, int norm,
+                    int nbits, int groups, half_t* __restrict__ logits, int* __restrict__ idx, half_t* __restrict__ w,
+                    int* __restrict__ hist_out) {
+  constexpr int EB = 4 * PER_LANE;             // blocks of 16 experts
+  constexpr int RR_THREADS = RR_WAVES * WAVE;
+  constexpr int EP = 16 * EB;                  // experts, padded
+  extern __shared__ __attribute__((aligned(16))) char lds_raw[];
+  float* part = reinterpret_cast<float*>(lds_raw);                      // [RR_WAVES][RR_TOKENS][EP]
+  half_t* lg = reinterpret_cast<half_t*>(part + RR_WAVES * RR_TOKENS * EP);  // [RR_TOKENS][EP]
+  int* sidx = reinterpret_cast<int*>(lg + RR_TOKENS * EP);              // [groups * RR_TOKENS * k]
+  int* hist = sidx + groups * RR_TOKENS * k;                           // [E]
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int row = lane & 15, kq = (lane >> 4) * 8;   // the operand row of this lane and its 8 halves of a K step
+  const int kwave = H / RR_WAVES, steps = kwave / RR_KSTEP;   // a multiple of 4 steps per wavefront
+  const __amdgpu_buffer_rsrc_t hrsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(h), 0, (int)((size_t)N * H * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rrsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(router), 0, (int)((size_t)E * H * 2), 0x00020000);
+
+  for (int g = 0; g < groups; ++g) {
+    const int t0 = (blockIdx.x * groups + g) * RR_TOKENS;
+    if (t0 < N) {
+      // ---- this wavefront's share of the dot products. Loads go through buffer descriptors: a
+      // token past N or an expert past E is out of range and reads as 0
+      const unsigned aoff = ((unsigned)(t0 + row) * (unsigned)H + (unsigned)(wave * kwave + kq)) * 2u;
+      const unsigned boff = ((unsigned)row * (unsigned)H + (unsigned)(wave * kwave + kq)) * 2u;
+      float4v_t acc[EB];
+#pragma unroll
+      for (int b = 0; b < EB; ++b) acc[b] = float4v_t{0.f, 0.f, 0.f, 0.f};
+      half8_t a0[2], a1[2], b0[2][EB], b1[2][EB];
+      auto load = [&](half8_t (&a)[2], half8_t (&bb)[2][EB], int s) {
+        // two steps are the two halves of a 128-byte line of each row: asked for one after the other
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+          a[u] = __builtin_bit_cast(half8_t, __builtin_amdgcn_raw_buffer_load_b128(hrsrc, aoff, (s + u) * RR_KSTEP * 2, 0));
+#pragma unroll
+        for (int b = 0; b < EB; ++b)
+#pragma unroll
+          for (int u = 0; u < 2; ++u)
+            bb[u][b] = __builtin_bit_cast(half8_t, __builtin_amdgcn_raw_buffer_load_b128(rrsrc, boff + (unsigned)(16 * b) * (unsigned)H * 2u,
+                                                                                        (s + u) * RR_KSTEP * 2, 0));
+      };
+      auto multiply = [&](const half8_t (&a)[2], const half8_t (&bb)[2][EB]) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int b = 0; b < EB; ++b) acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[u], bb[u][b], acc[b], 0, 0, 0);
+      };
+      load(a0, b0, 0);
+      for (int s = 0; s < steps; s += 4) {
+        load(a1, b1, s + 2);
+        multiply(a0, b0);
+        if (s + 4 < steps) load(a0, b0, s + 4);
+        multiply(a1, b1);
+      }
+      // lane holds tokens 4 * (lane / 16) + r, expert 16 b + lane % 16
+#pragma unroll
+      for (int b = 0; b < EB; ++b)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) part[(wave * RR_TOKENS + 4 * (lane >> 4) + r) * EP + 16 * b + row] = acc[b][r];
+    }
+    __syncthreads();
+    if (t0 < N) {
+      for (int o = tid; o < RR_TOKENS * EP; o += RR_THREADS) {
+        const int tok = o / EP, e = o - tok * EP;
+        float v = part[o];
+#pragma unroll
+        for (int q = 1; q < RR_WAVES; ++q) v += part[q * RR_TOKENS * EP + o];
+        const half_t hv = (half_t)v;
+        lg[o] = hv;
+        if (t0 + tok < N && e < E) logits[(size_t)(t0 + tok) * E + e] = hv;
+      }
+    }
+    __syncthreads();
+    // ---- route: one wavefront per token
+    for (int tok = wave; tok < RR_TOKENS; tok += RR_WAVES) {
+      const int t = t0 + tok;
+      int my_e = -1;
+      if (t < N) {
+        float my_w;
+        route_core::route_token<half_t, PER_LANE>(lg + tok * EP, E, k, norm, my_e, my_w);
+        if (lane < k) {
+          idx[(size_t)t * k + lane] = my_e;
+          w[(size_t)t * k + lane] = (half_t)my_w;
+        }
+      }
+      if (lane < k) sidx[(g * RR_TOKENS + tok) * k + lane] = my_e;
+    }
+  }
+  if (!hist_out) return;
+  __syncthreads();
+  // ---- the workgroup's choices are one piece of the sort: their histogram
+  if (wave == 0) {
+    for (int e = lane; e < E; e += WAVE) hist[e] = 0;
+    count_piece(sidx, 0, groups * RR_TOKENS * k, E, nbits, hist);
+    for (int e = lane; e < E; e += WAVE) hist_out[(size_t)blockIdx.x * E + e] = hist[e];
+  }
+}
+
+bool router_route_shape_ok(int N, int H, int E, int k) {
+  return N >= 1 && H >= 512 && H % 512 == 0 && E >= 1 && E <= 128 && k >= 1 && k <= FRONT_MAX_K && k <= E &&
+         (long)N * H * 2 < (1l << 31);
+}
+
+int launch_router_route(const void* h, const void* router, int N, int H, int E, int k, int norm, void* logits,
+                        int32_t* idx, void* w, void* hist, hipStream_t st) {
+  int nbits = 0;
+  while ((1 << nbits) < E) ++nbits;
+  const long M = (long)N * k;
+  int groups = 1, grid = (N + RR_TOKENS - 1) / RR_TOKENS;
+  if (hist) {   // one workgroup per piece of the sort, and as many pieces as its second launch reads
+    groups = piece_for(M) / (RR_TOKENS * k);
+    grid = large_blocks(M) * SORT_WAVES;
+  }
+  const int EP = E <= 64 ? 64 : 128;
+  const bool wide = E <= 64 && H % 2048 == 0;   // 16 wavefronts: four K steps each at H = 2048
+  const int waves = wide ? 16 : 4;
+  const size_t lds = sizeof(float) * waves * RR_TOKENS * EP + sizeof(half_t) * RR_TOKENS * EP +
+                     sizeof(int) * ((size_t)groups * RR_TOKENS * k + E);
+  void (*kern)(const half_t*, const half_t*, int, int, int, int, int, int, int, half_t*, int*, half_t*, int*) =
+      wide ? router_route_kernel<1, 16> : E <= 64 ? router_route_kernel<1, 4> : router_route_kernel<2, 4>;
+  if (lds > 48 * 1024 && hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+    return sy_fail(SY_ERR_LAUNCH, "router_route: cannot reserve %zu bytes of LDS", lds);
+  kern<<<grid, waves * WAVE, lds, st>>>((const half_t*)h, (const half_t*)router, N, H, E, k, norm, nbits, groups,
+                                        (half_t*)logits, idx, (half_t*)w, (int*)hist);
+  return sy_check_launch("router_route");
+}
+
 }  // namespace
 
 extern "C" SY_API int sy_route_sort(const void* logits, int N, int E, int k, int norm, int32_t* idx, void* w,
@@ -80,4 +232,26 @@ extern "C" SY_API int sy_route_sort(const void* logits, int N, int E, int k, int
     front_kernel<2><<<1, threads, lds, st>>>((const half_t*)logits, N, E, k, norm, nbits, idx, (half_t*)w, counts,
                                                   offsets, token, (half_t*)wsorted, pos_of);
   return sy_check_launch("route_sort");
+}
+
+// Whether the router + route launch can also be the sort's first pass: the sort runs over many
+// workgroups (above the one-workgroup limit) and a piece is whole groups of 16 tokens.
+bool sy_router_route_counts(int N, int k) {
+  const long M = (long)N * k;
+  return M > SMALL_M && piece_for(M) % (RR_TOKENS * k) == 0;
+}
+
+int sy_router_route_counting(const void* h, const void* router, int N, int H, int E, int k, int norm, void* logits,
+                             int32_t* idx, void* w, void* hist, void* stream) {
+  SY_REQUIRE(router_route_shape_ok(N, H, E, k),
+             "router_route: H a multiple of 512, at most 128 experts and top-8 (got N = %d, H = %d, E = %d, k = %d)", N, H, E, k);
+  SY_REQUIRE(h && router && logits && idx && w, "router_route: null pointer");
+  SY_REQUIRE(!hist || sy_router_route_counts(N, k), "router_route: no histograms for N = %d, k = %d", N, k);
+  return launch_router_route(h, router, N, H, E, k, norm, logits, idx, w, hist, (hipStream_t)stream);
+}
+
+extern "C" SY_API int sy_router_route(const void* h, const void* router, int N, int H, int E, int k, int norm, void* logits,
+                                      int32_t* idx, void* w, void* stream) {
+  if (N == 0) return SY_OK;
+  return sy_router_route_counting(h, router, N, H, E, k, norm, logits, idx, w, nullptr, stream);
 }

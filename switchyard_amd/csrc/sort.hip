@@ -148,21 +148,9 @@ int bits_for(int E) {
   return b;
 }
 
-// Choices per wavefront in the launches over many workgroups. A wavefront walks its piece 64
-// choices at a time and every step is a chain of a load, ballots and scattered stores, so
-// short pieces on many CUs finish sooner (32 768 choices: 23 us with pieces of 512 on 4 CUs);
-// long inputs take longer pieces so that the table of histograms, which every workgroup of the
-// second launch reads in full, stays small.
-int piece_for(long M) { return M <= 65536 ? 128 : M <= 262144 ? 256 : PIECE; }
-
-int large_blocks(long M) {
-  const long per_block = (long)piece_for(M) * SORT_WAVES;
-  return (int)((M + per_block - 1) / per_block);
-}
-
 template <typename W>
 int launch_sort(const int32_t* idx, const void* w, int M, int k, int E, int32_t* counts, int32_t* offsets,
-                int32_t* token, void* wsorted, int32_t* pos_of, void* workspace, hipStream_t stream) {
+                int32_t* token, void* wsorted, int32_t* pos_of, void* workspace, hipStream_t stream, bool counted = false) {
   const int nbits = bits_for(E);
   if (M <= SMALL_M) {
     const size_t lds = sizeof(int) * small_sort_lds_ints(E);
@@ -172,8 +160,10 @@ int launch_sort(const int32_t* idx, const void* w, int M, int k, int E, int32_t*
   }
   const int blocks = large_blocks(M), nvirtual = blocks * SORT_WAVES;
   const int piece = piece_for(M);
-  sort_count_kernel<<<blocks, SORT_THREADS, sizeof(int) * SORT_WAVES * E, stream>>>(idx, M, E, nbits, piece, (int*)workspace);
-  if (int rc = sy_check_launch("sort_by_expert (count)")) return rc;
+  if (!counted) {
+    sort_count_kernel<<<blocks, SORT_THREADS, sizeof(int) * SORT_WAVES * E, stream>>>(idx, M, E, nbits, piece, (int*)workspace);
+    if (int rc = sy_check_launch("sort_by_expert (count)")) return rc;
+  }
   const size_t lds = sizeof(int) * ((size_t)SORT_WAVES * E + 2 * SORT_THREADS + 3 * E + 1 + SORT_WAVES);
   sort_assign_kernel<W><<<blocks, SORT_THREADS, lds, stream>>>(idx, (const W*)w, M, k, E, nbits, piece, (const int*)workspace,
                                                                nvirtual, counts, offsets, token, (W*)wsorted, pos_of);
@@ -181,6 +171,13 @@ int launch_sort(const int32_t* idx, const void* w, int M, int k, int E, int32_t*
 }
 
 }  // namespace
+
+// The second launch alone, for a caller whose own kernel has left the per-piece histograms in the
+// workspace (the router + route launch of front.hip). Weights of 2 bytes; N*k above SMALL_M.
+int sy_sort_assign_counted(const int32_t* idx, const void* w, int N, int k, int E, int32_t* counts, int32_t* offsets,
+                           int32_t* token, void* wsorted, int32_t* pos_of, void* workspace, void* stream) {
+  return launch_sort<uint16_t>(idx, w, N * k, k, E, counts, offsets, token, wsorted, pos_of, workspace, (hipStream_t)stream, true);
+}
 
 extern "C" SY_API size_t sy_sort_workspace_bytes(int N, int k, int E) {
   const long M = (long)N * k;

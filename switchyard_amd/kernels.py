@@ -37,8 +37,18 @@ def tile_offsets(counts, block=64):
     return off
 
 
+# From this many tokens on the router GEMM and route are one launch of this library (the
+# library GEMM for 64 output columns takes about 14 us at any of these sizes, the route launch 6).
+ROUTER_ROUTE_MIN_TOKENS = 65
+
+
 def route(h, router, top_k, norm_topk_prob):
     """Returns (indices int32 [N, k], weights in h's dtype [N, k]); ties go to the lower expert id."""
+    N, H = h.shape
+    if (N >= ROUTER_ROUTE_MIN_TOKENS and h.dtype == torch.float16 and router.dtype == torch.float16
+            and _abi.Ext.router_route_ok(N, H, router.shape[0], top_k)):
+        idx, w, _ = ext().router_route(h.contiguous(), router.contiguous(), top_k, norm_topk_prob)
+        return idx, w
     return ext().route(F.linear(h, router).contiguous(), top_k, norm_topk_prob)
 
 
@@ -181,7 +191,10 @@ def moe_layer(h, router, gate_up, down, top_k, norm_topk_prob, mode="auto"):
             mode = _auto(N, N * top_k, n_experts)
         if mode not in ("gemv", "gemm", "cublas"):
             raise ValueError(f"unknown mode {mode!r}")
-        own = N <= OWN_ROUTER_MAX_TOKENS and h.shape[1] % 8 == 0 and h.shape[1] <= 8192
+        if N <= OWN_ROUTER_MAX_TOKENS:
+            own = h.shape[1] % 8 == 0 and h.shape[1] <= 8192
+        else:   # the router GEMM, route and the sort's first pass in one launch
+            own = router.dtype == torch.float16 and _abi.Ext.router_route_ok(N, h.shape[1], n_experts, top_k)
         return ext().moe_experts(h.contiguous(), None if own else F.linear(h, router).contiguous(), gate_up, down, top_k,
                                  norm_topk_prob, mfma_tiles=mode != "gemv", one_launch_front=N <= FUSED_FRONT_MAX_TOKENS,
                                  router=router.contiguous() if own else None)

@@ -305,9 +305,10 @@ def test_a_step_on_the_decode_kernels_gives_the_logits_of_the_torch_step(batch, 
     # within a rounding of each other, the two may pick different experts, and that (step, sequence)
     # then differs by more than rounding. Such near-ties are rare (about one decision in a hundred;
     # 1 of the 192 pairs at 64 sequences), so at most 2 % of the (step, sequence) pairs may exceed
-    # the tolerance, and none by much.
+    # the tolerance (one pair where 2 % is less than one: which roundings meet a near-tie changes
+    # with every change to a kernel's order of summation, at any batch size), and none by much.
     per = (logits[0].float() - logits[1].float()).abs().amax(-1)            # [steps, B]
-    allowed = per.numel() // 50
+    allowed = max(1, per.numel() // 50)
     assert int((per > 2e-2).sum()) <= allowed, per.amax(0)
     assert per.max().item() < 0.3
     for a, b in ((caches[0].k, caches[1].k), (caches[0].v, caches[1].v)):

@@ -440,10 +440,48 @@ def test_route_sort_limits(K):
         K.ext().route_sort(torch.zeros(4, 64, dtype=torch.float16, device=DEV), 9, False)
 
 
+@pytest.mark.parametrize("N,E,k,H", [(65, 64, 8, 2048), (1000, 64, 8, 2048), (4096, 64, 8, 2048), (77, 128, 8, 512),
+                                     (333, 100, 5, 1024), (16, 8, 2, 512), (1, 64, 8, 512)])
+@pytest.mark.parametrize("norm", [False, True])
+def test_router_gemm_and_route_in_one_launch(K, N, E, k, H, norm):
+    """sy_router_route: logits as the GEMM gives them (to half-precision rounding), and from
+    those logits exactly route's ids and weights, which are the oracle's."""
+    g = torch.Generator().manual_seed(N + E)
+    h = torch.randn(N, H, generator=g).half().to(DEV)
+    router = (torch.randn(E, H, generator=g) * H ** -0.5).half().to(DEV)
+    idx, w, logits = K.ext().router_route(h, router, k, norm)
+    assert torch.allclose(logits.float(), h.float() @ router.float().T, rtol=2 ** -10, atol=1e-3)
+    ridx, rw = K.ext().route(logits, k, norm)
+    assert torch.equal(idx, ridx) and torch.equal(w, rw)
+    oidx, ow = O.route_logits(logits.cpu(), k, norm)
+    assert torch.equal(idx.cpu().long(), oidx)
+    assert (w.cpu().float() - ow.float()).abs().max().item() < WEIGHT_TOL
+    if N >= K.ROUTER_ROUTE_MIN_TOKENS:   # kernels.route takes this launch from there on
+        kidx, kw = K.route(h, router, k, norm)
+        assert torch.equal(kidx, idx) and torch.equal(kw, w)
+
+
+def test_router_route_limits(K):
+    h = torch.zeros(100, 768, dtype=torch.float16, device=DEV)
+    with pytest.raises(RuntimeError):
+        K.ext().router_route(h, torch.zeros(64, 768, dtype=torch.float16, device=DEV), 8, False)   # H % 512 != 0
+    h = torch.zeros(100, 512, dtype=torch.float16, device=DEV)
+    with pytest.raises(RuntimeError):
+        K.ext().router_route(h, torch.zeros(200, 512, dtype=torch.float16, device=DEV), 8, False)  # too many experts
+    # a layer of that width still runs: the library GEMM makes the logits
+    hh, router, gu, dn = (t.to(DEV) for t in cases.layer(100, E=16, k=4, H=768, I=64, seed=1, wstd=0.05))
+    out = K.moe_layer(hh, router, gu, dn, 4, False)
+    assert out.shape == (100, 768) and torch.isfinite(out.float()).all()
+
+
 # ------------------------------------------------------------------ the experts of a decode step in one call
 @pytest.mark.parametrize("N,E,k,H,I", [(1, 64, 8, 2048, 1024), (8, 64, 8, 2048, 1024), (16, 64, 8, 2048, 1024),
                                        (5, 16, 4, 128, 64), (40, 64, 8, 256, 128), (200, 64, 8, 256, 128),
-                                       (3000, 64, 8, 128, 64)])        # the sort with a workspace
+                                       (3000, 64, 8, 128, 64),         # the sort with a workspace
+                                       # router GEMM and route in one launch (H a multiple of 512, above 64 tokens):
+                                       (100, 64, 8, 512, 128), (300, 128, 8, 512, 64),
+                                       # ... which is also the sort's first pass above 8192 choices
+                                       (1100, 64, 8, 512, 64), (2100, 16, 4, 512, 64), (1027, 60, 8, 1024, 64)])
 @pytest.mark.parametrize("tiles", [False, True])
 @pytest.mark.parametrize("norm", [False, True])
 def test_experts_in_one_call_equal_the_five_calls(K, N, E, k, H, I, tiles, norm):
@@ -454,7 +492,11 @@ def test_experts_in_one_call_equal_the_five_calls(K, N, E, k, H, I, tiles, norm)
     h, router, gu, dn = (t.to(DEV) for t in (h, router, gu, dn))
     ext = K.ext()
     # the logits the layer itself will route on: the library's own router kernel for tens of tokens
-    logits = ext.router_logits(h, router) if N <= K.OWN_ROUTER_MAX_TOKENS else F.linear(h, router).contiguous()
+    fused_router = N > K.OWN_ROUTER_MAX_TOKENS and ext.router_route_ok(N, H, E, k)
+    if fused_router:
+        fidx, fw, logits = ext.router_route(h, router, k, norm)
+    else:
+        logits = ext.router_logits(h, router) if N <= K.OWN_ROUTER_MAX_TOKENS else F.linear(h, router).contiguous()
     assert torch.allclose(logits.float(), h.float() @ router.float().T, rtol=2 ** -10, atol=1e-4)
     one_launch = N <= K.FUSED_FRONT_MAX_TOKENS
     if one_launch:
@@ -462,6 +504,8 @@ def test_experts_in_one_call_equal_the_five_calls(K, N, E, k, H, I, tiles, norm)
     else:
         idx, w = ext.route(logits, k, norm)
         counts, offsets, token, wsorted, pos_of = ext.sort_by_expert(idx, w, E)
+    if fused_router:   # the launch that made the logits routed on them as route does
+        assert torch.equal(fidx, idx) and torch.equal(fw, w)
     M = N * k
     if tiles:
         act = ext.grouped_gemm(h, token, gu, offsets, None, 0, M, True, None)
@@ -474,6 +518,6 @@ def test_experts_in_one_call_equal_the_five_calls(K, N, E, k, H, I, tiles, norm)
     assert torch.equal(got, want)
     layer = K.moe_layer(h, router, gu, dn, k, norm, mode="gemm" if tiles else "gemv")   # the layer takes this path
     assert torch.equal(layer, want)
-    if N <= K.OWN_ROUTER_MAX_TOKENS:     # and with the router GEMM inside the same call
+    if N <= K.OWN_ROUTER_MAX_TOKENS or fused_router:     # and with the router GEMM inside the same call
         assert torch.equal(ext.moe_experts(h, None, gu, dn, k, norm, mfma_tiles=tiles, one_launch_front=one_launch,
                                            router=router), want)
