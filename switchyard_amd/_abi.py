@@ -104,8 +104,13 @@ _DTYPE_CODE = {torch.float16: 0, torch.float32: 1}
 class Ext:
     """The native module: route, sort_by_expert, grouped_gemv, grouped_gemm, combine."""
 
+    PLAN_BYTES_MAX = 32 << 20   # moe_experts keeps the scratch of calls up to this size ...
+    PLANS_MAX = 16              # ... for this many (shape, stream) pairs
+    EARLY_LOGITS = True
+
     def __init__(self, lib=None):
         self.lib = lib or load_library()
+        self._plans = {}
 
     def _call(self, fn, *args):
         rc = fn(*args)
@@ -233,22 +238,46 @@ class Ext:
                 raise RuntimeError("moe_experts: router must be [E, H]")
         if tuple(gate_up.shape) != (E, 2 * I, H) or tuple(down.shape) != (E, H, I):
             raise RuntimeError("moe_experts: shapes of h / gate_up / down do not match")
-        M = N * int(k)
-        need = 0 if one_launch_front else self.lib.sy_sort_workspace_bytes(N, int(k), E)
-        # idx w counts offsets token wsorted pos_of act y, then the sort's workspace and the logits
-        sizes = [M * 4, M * 2, E * 4, (E + 1) * 4, M * 4, M * 2, M * 4, M * I * 2, M * H * 2, need,
-                 N * E * 2 if logits is None else 0]
-        starts, at = [], 0
-        for size in sizes:
-            starts.append(at)
-            at += (size + 255) // 256 * 256
-        scratch = torch.empty(at, dtype=torch.uint8, device=h.device)
-        out = torch.empty((N, H), dtype=torch.float16, device=h.device)
+        stream = _stream()
+        # The intermediate results of small calls (a decode step's) live in an allocation that is
+        # kept per shape and stream: calls on one stream run in order, so they may share it, and a
+        # call once waited for is timed with this function's host time in front of its first launch.
+        key = (N, E, int(k), H, I, logits is None, bool(one_launch_front), h.device.index, stream)
+        plan = self._plans.get(key)
+        if plan is None:
+            M = N * int(k)
+            need = 0 if one_launch_front else self.lib.sy_sort_workspace_bytes(N, int(k), E)
+            # idx w counts offsets token wsorted pos_of act y, then the sort's workspace and the logits
+            sizes = [M * 4, M * 2, E * 4, (E + 1) * 4, M * 4, M * 2, M * 4, M * I * 2, M * H * 2, need,
+                     N * E * 2 if logits is None else 0]
+            starts, at = [], 0
+            for size in sizes:
+                starts.append(at)
+                at += (size + 255) // 256 * 256
+            plan = (starts, at, need, None)
+            if at <= self.PLAN_BYTES_MAX:
+                if len(self._plans) >= self.PLANS_MAX:
+                    self._plans.pop(next(iter(self._plans)))
+                plan = (starts, at, need, torch.empty(at, dtype=torch.uint8, device=h.device))
+                self._plans[key] = plan
+        starts, at, need, scratch = plan
+        if scratch is None:
+            scratch = torch.empty(at, dtype=torch.uint8, device=h.device)
         base = scratch.data_ptr()
-        self._call(self.lib.sy_moe_experts, h.data_ptr(), router.data_ptr() if router is not None else None,
+        router_ptr = router.data_ptr() if router is not None else None
+        if router is not None and N <= 64 and self.EARLY_LOGITS:
+            # the router's logits are enqueued at once: the GPU works on them while the host
+            # allocates the result and marshals the long call (a call that is waited for starts
+            # its first kernel 4 us sooner; in a stream of calls nothing changes)
+            self._call(self.lib.sy_router_logits, h.data_ptr(), router_ptr, N, H, E, base + starts[10], stream)
+            router_ptr = None
+        out = torch.empty((N, H), dtype=torch.float16, device=h.device)
+        self._call(self.lib.sy_moe_experts, h.data_ptr(), router_ptr,
                    logits.data_ptr() if logits is not None else base + starts[10], N, E, int(k), int(bool(norm)),
                    gate_up.data_ptr(), down.data_ptr(), H, I, int(bool(mfma_tiles)), int(bool(one_launch_front)),
-                   *[base + s for s in starts[:9]], out.data_ptr(), base + starts[9] if need else None, need, _stream())
+                   base + starts[0], base + starts[1], base + starts[2], base + starts[3], base + starts[4], base + starts[5],
+                   base + starts[6], base + starts[7], base + starts[8], out.data_ptr(), base + starts[9] if need else None,
+                   need, stream)
         return out
 
     @staticmethod
