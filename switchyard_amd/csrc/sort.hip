@@ -100,6 +100,30 @@ sort_assign_kernel(const int* __restrict__ idx, const W* __restrict__ w, int M, 
   int* tmp = offs + E + 1;                 // [SORT_WAVES]
   const int t = threadIdx.x, wv = t >> 6;
   const int v0 = blockIdx.x * SORT_WAVES;
+  const long lo64 = (long)(v0 + wv) * piece;
+  const int lo = (int)(lo64 < M ? lo64 : M), hi = min(lo + piece, M);
+
+  // Everything this workgroup reads that does not depend on the scan is asked for first: its
+  // own wavefronts' histograms, and (pieces of two groups) the keys and weights it will
+  // scatter. The kernel is a chain of memory round trips around little work; this makes it one.
+  const bool loaded = piece == 2 * WAVE;
+  int keys[2] = {-1, -1};
+  W weights[2] = {0, 0};
+  if (loaded) {
+#pragma unroll
+    for (int g = 0; g < 2; ++g) {
+      const int i = lo + g * WAVE + (t & 63);
+      if (i < hi) {
+        keys[g] = idx[i];
+        weights[g] = w[i];
+      }
+    }
+  }
+  int own[SORT_WAVES];
+  if (t < E) {
+#pragma unroll
+    for (int j = 0; j < SORT_WAVES; ++j) own[j] = v0 + j < nvirtual ? ws[(size_t)(v0 + j) * E + t] : 0;
+  }
 
   // thread (part, e): sums ws[v][e] over v = part, part + parts, ...
   const int parts = SORT_THREADS / E;  // >= 1 because E <= 1024
@@ -131,15 +155,15 @@ sort_assign_kernel(const int* __restrict__ idx, const W* __restrict__ w, int M, 
     for (int j = t; j <= E; j += SORT_THREADS) offsets[j] = offs[j];
   if (t < E) {
     int run = offs[t] + before[t];
+#pragma unroll
     for (int j = 0; j < SORT_WAVES; ++j) {
       base[j * E + t] = run;
-      if (v0 + j < nvirtual) run += ws[(size_t)(v0 + j) * E + t];
+      run += own[j];
     }
   }
   __syncthreads();
-  const long lo64 = (long)(v0 + wv) * piece;
-  const int lo = (int)(lo64 < M ? lo64 : M), hi = min(lo + piece, M);
-  assign_piece(idx, w, lo, hi, k, E, nbits, base + wv * E, token, wsorted, pos_of);
+  if (loaded) assign_loaded(keys, weights, lo, k, E, nbits, base + wv * E, token, wsorted, pos_of);
+  else assign_piece(idx, w, lo, hi, k, E, nbits, base + wv * E, token, wsorted, pos_of);
 }
 
 int bits_for(int E) {

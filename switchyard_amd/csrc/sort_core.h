@@ -98,6 +98,35 @@ __device__ __forceinline__ void scan_experts(const int* total, int E, int* offs,
 // small_sort_lds_ints(E) ints. idx and w may live in global memory or in LDS.
 __host__ __device__ constexpr size_t small_sort_lds_ints(int E) { return (size_t)SORT_WAVES * E + 2 * E + 1 + SORT_WAVES; }
 
+// The same for a piece of two groups of 64 whose keys and weights the caller has already loaded
+// (key -1 where the piece has no choice): the loads were issued before the histograms were
+// summed, so nothing here waits for memory before it scatters.
+template <typename W>
+__device__ __forceinline__ void assign_loaded(const int (&keys)[2], const W (&weights)[2], int lo, int k, int E, int nbits,
+                                              int* base, int* __restrict__ token, W* __restrict__ wsorted,
+                                              int* __restrict__ pos_of) {
+  const int lane = threadIdx.x & 63;
+#pragma unroll
+  for (int g = 0; g < 2; ++g) {
+    const int i = lo + g * WAVE + lane;
+    int key = keys[g];
+    const bool valid = (unsigned)key < (unsigned)E;
+    key = valid ? key : 0;
+    const uint64_t m = match_lanes(key, valid, nbits);
+    const int rank = __popcll(m & lanemask_lt()), cnt = __popcll(m);
+    int row = 0;
+    if (valid) row = base[key] + rank;
+    __builtin_amdgcn_wave_barrier();
+    if (valid) {
+      token[row] = i / k;
+      wsorted[row] = weights[g];
+      pos_of[i] = row;
+      if (rank == cnt - 1) base[key] += cnt;
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
 template <typename W>
 __device__ __forceinline__ void sort_small_block(const int* idx, const W* w, int M, int k, int E, int nbits,
                                                  int* __restrict__ counts, int* __restrict__ offsets,
