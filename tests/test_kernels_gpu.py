@@ -481,7 +481,9 @@ def test_router_route_limits(K):
                                        # router GEMM and route in one launch (H a multiple of 512, above 64 tokens):
                                        (100, 64, 8, 512, 128), (300, 128, 8, 512, 64),
                                        # ... which is also the sort's first pass above 8192 choices
-                                       (1100, 64, 8, 512, 64), (2100, 16, 4, 512, 64), (1027, 60, 8, 1024, 64)])
+                                       (1100, 64, 8, 512, 64), (2100, 16, 4, 512, 64), (1027, 60, 8, 1024, 64),
+                                       # ... with two and four groups of 16 tokens to a piece of the sort
+                                       (9000, 64, 8, 512, 64), (33000, 64, 8, 512, 32)])
 @pytest.mark.parametrize("tiles", [False, True])
 @pytest.mark.parametrize("norm", [False, True])
 def test_experts_in_one_call_equal_the_five_calls(K, N, E, k, H, I, tiles, norm):
