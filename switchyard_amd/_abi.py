@@ -10,6 +10,7 @@ GIL around every call, as the reference's call guards do.
 There is no fallback: if the library is missing and cannot be built, loading raises."""
 
 import ctypes
+import threading
 import os
 
 import torch
@@ -111,6 +112,7 @@ class Ext:
     def __init__(self, lib=None):
         self.lib = lib or load_library()
         self._plans = {}
+        self._plans_lock = threading.Lock()
 
     def _call(self, fn, *args):
         rc = fn(*args)
@@ -263,6 +265,18 @@ class Ext:
         starts, at, need, scratch = plan
         if scratch is None:
             scratch = torch.empty(at, dtype=torch.uint8, device=h.device)
+            return self._enqueue_experts(h, router, logits, gate_up, down, k, norm, mfma_tiles, one_launch_front,
+                                         scratch, starts, need, stream)
+        # kept scratch: two threads enqueueing the same shape on one stream must not interleave
+        # their launches (ctypes releases the GIL inside the calls)
+        with self._plans_lock:
+            return self._enqueue_experts(h, router, logits, gate_up, down, k, norm, mfma_tiles, one_launch_front,
+                                         scratch, starts, need, stream)
+
+    def _enqueue_experts(self, h, router, logits, gate_up, down, k, norm, mfma_tiles, one_launch_front, scratch, starts,
+                         need, stream):
+        N, H = h.shape
+        E, I = gate_up.shape[0], down.shape[2]
         base = scratch.data_ptr()
         router_ptr = router.data_ptr() if router is not None else None
         if router is not None and N <= 64 and self.EARLY_LOGITS:
