@@ -107,7 +107,6 @@ class Ext:
 
     PLAN_BYTES_MAX = 32 << 20   # moe_experts keeps the scratch of calls up to this size ...
     PLANS_MAX = 16              # ... for this many (shape, stream) pairs
-    EARLY_LOGITS = True
 
     def __init__(self, lib=None):
         self.lib = lib or load_library()
@@ -279,7 +278,7 @@ class Ext:
         E, I = gate_up.shape[0], down.shape[2]
         base = scratch.data_ptr()
         router_ptr = router.data_ptr() if router is not None else None
-        if router is not None and N <= 64 and self.EARLY_LOGITS:
+        if router is not None and N <= 64:
             # the router's logits are enqueued at once: the GPU works on them while the host
             # allocates the result and marshals the long call (a call that is waited for starts
             # its first kernel 4 us sooner; in a stream of calls nothing changes)
