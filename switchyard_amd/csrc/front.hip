@@ -179,6 +179,161 @@ router_route_kernel(const half_t* __restrict__ h, const half_t* __restrict__ rou
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// The same launch with the operands staged through LDS, for up to 64 experts. What the kernel
+// above waits for is its compute unit's L1: every workgroup pulls the whole router through it, and
+// an MFMA operand load takes a 64-byte piece of each of 16 rows, which costs the L1 what a whole
+// line costs. Here the router's rows and the workgroup's 16 token rows come in K slices of 64
+// (128 bytes of a row: whole lines, 8 rows per instruction) by buffer loads that write LDS
+// directly, fourteen slices deep, so 130 KB of loads are in flight while one slice is multiplied
+// (with eight slices the loop waited for data in every iteration: 11.0 us a launch against 9);
+// a slice's 16-byte chunks are XOR-swizzled by row so that the operand reads spread over the
+// banks. Ten wavefronts issue one load per slice each (eight the router's rows, two the
+// tokens'), eight multiply (expert block x half of the slice's K), all sixteen route. The waits
+// for the loads are counted by hand: the compiler is not told about them.
+constexpr int RS_WAVES = 16, RS_THREADS = RS_WAVES * WAVE, RS_DEPTH = 14;   // 140 of the 160 KB of LDS are slices
+constexpr int RS_ROWS = 64 + RR_TOKENS, RS_STAGE = RS_ROWS * 128, RS_LOADS = RS_ROWS / 8;
+constexpr int RS_BK = 64;
+
+typedef int int4v_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ int4v_t raw_descriptor(const void* base, unsigned bytes) {
+  const uint64_t a = (uint64_t)base;
+  int4v_t d;
+  d[0] = __builtin_amdgcn_readfirstlane((int)(unsigned)a);
+  d[1] = __builtin_amdgcn_readfirstlane((int)((unsigned)(a >> 32) & 0xffffu));
+  d[2] = __builtin_amdgcn_readfirstlane((int)bytes);
+  d[3] = 0x00020000;
+  return d;
+}
+
+// 16 bytes per lane from buffer offset voffset + soffset to LDS address lds_addr + 16 * lane;
+// only voffset is checked against the size of the buffer. The LDS address travels in m0.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+__device__ __forceinline__ void buffer_to_lds(int4v_t rsrc, unsigned voffset, unsigned soffset, unsigned lds_addr) {
+#pragma unroll
+  for (int c = 0; c < 4; ++c) rsrc[c] = __builtin_amdgcn_readfirstlane(rsrc[c]);
+  soffset = __builtin_amdgcn_readfirstlane(soffset);
+  lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "buffer_load_dwordx4 %1, %2, %3 offen lds"
+      :
+      : "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset)
+      : "memory", "m0");
+}
+#pragma clang diagnostic pop
+
+__global__ void __launch_bounds__(RS_THREADS)
+router_route_staged_kernel(const half_t* __restrict__ h, const half_t* __restrict__ router, int N, int H, int E, int k,
+                           int norm, int nbits, int groups, half_t* __restrict__ logits, int* __restrict__ idx,
+                           half_t* __restrict__ w, int* __restrict__ hist_out) {
+  constexpr int EP = 64;
+  constexpr unsigned OUT_OF_RANGE = 0x80000000u;
+  extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
+  float* part = reinterpret_cast<float*>(lds_raw + RS_DEPTH * RS_STAGE);   // [2][RR_TOKENS][EP]
+  half_t* lg = reinterpret_cast<half_t*>(part + 2 * RR_TOKENS * EP);      // [RR_TOKENS][EP]
+  int* sidx = reinterpret_cast<int*>(lg + RR_TOKENS * EP);                // [groups * RR_TOKENS * k]
+  int* hist = sidx + groups * RR_TOKENS * k;                             // [E]
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int nk = H / RS_BK;
+  const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) char*)lds_raw;
+  const int4v_t rrsrc = raw_descriptor(router, (unsigned)((size_t)E * H * 2));
+  const int4v_t hrsrc = raw_descriptor(h, (unsigned)((size_t)N * H * 2));
+  const bool loads = wave < RS_LOADS, multiplies = wave < 8;
+  // a multiplying wavefront: expert block and which half of a slice's K
+  const int block = wave & 3, khalf = (wave >> 2) & 1;
+  const int orow = lane & 15, ochunk = 4 * khalf + (lane >> 4);
+  const int arow = 64 + orow, brow = 16 * block + orow;
+  const unsigned aread = arow * 128 + ((ochunk ^ ((arow >> 1) & 7)) * 16), bread = brow * 128 + ((ochunk ^ ((brow >> 1) & 7)) * 16);
+
+  for (int g = 0; g < groups; ++g) {
+    const int t0 = (blockIdx.x * groups + g) * RR_TOKENS;
+    if (t0 < N) {
+      // the row of the stage that this lane fetches a chunk of (rows 0..63 the router's, 64..79 the tokens')
+      const int srow = 8 * wave + (lane >> 3);
+      const unsigned chunk = (unsigned)((lane & 7) ^ ((srow >> 1) & 7));
+      unsigned voff = OUT_OF_RANGE;
+      if (wave < 8) {
+        if (srow < E) voff = ((unsigned)srow * (unsigned)H + chunk * 8u) * 2u;
+      } else if (loads) {
+        const int t = t0 + srow - 64;
+        if (t < N) voff = ((unsigned)t * (unsigned)H + chunk * 8u) * 2u;
+      }
+      // slices past the end are asked for too, out of range: they keep the count of loads in flight
+      // the same in every iteration and bring nothing
+      auto issue = [&](int s, int stage) {
+        if (loads)
+          buffer_to_lds(wave < 8 ? rrsrc : hrsrc, s < nk ? voff : OUT_OF_RANGE, (unsigned)s * (RS_BK * 2),
+                        lds_base + (unsigned)stage * RS_STAGE + (unsigned)wave * 1024u);
+      };
+      for (int s = 0; s < RS_DEPTH - 2; ++s) issue(s, s);
+      float4v_t acc = {0.f, 0.f, 0.f, 0.f};
+      int at = 0, fill = RS_DEPTH - 2;   // the buffer of slice s, and the one the next load fills
+      // two slices to a barrier (the number of slices is even: H is a multiple of 512)
+      for (int s = 0; s < nk; s += 2) {
+        // this wavefront's loads of slices s and s + 1 have landed when only the RS_DEPTH - 4 after them are in flight
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(RS_DEPTH - 4) : "memory");
+        __syncthreads();   // everybody's have; and everybody has read slices s - 2 and s - 1, whose buffers the next loads fill
+        const int at1 = at + 1, fill1 = fill + 1 == RS_DEPTH ? 0 : fill + 1;
+        issue(s + RS_DEPTH - 2, fill);
+        issue(s + RS_DEPTH - 1, fill1);
+        if (multiplies) {
+          const char* stage = lds_raw + at * RS_STAGE;
+          const half8_t a0 = *reinterpret_cast<const half8_t*>(stage + aread);
+          const half8_t b0 = *reinterpret_cast<const half8_t*>(stage + bread);
+          const half8_t a1 = *reinterpret_cast<const half8_t*>(stage + RS_STAGE + aread);
+          const half8_t b1 = *reinterpret_cast<const half8_t*>(stage + RS_STAGE + bread);
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, b0, acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, b1, acc, 0, 0, 0);
+        }
+        fill = at;   // slices s and s + 1 sit in buffers at, at + 1 (RS_DEPTH is even: pairs never wrap inside)
+        at = at1 + 1 == RS_DEPTH ? 0 : at1 + 1;
+      }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      // lane holds tokens 4 * (lane / 16) + r, expert 16 * block + lane % 16, for its half of every slice
+      if (multiplies) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) part[(khalf * RR_TOKENS + 4 * (lane >> 4) + r) * EP + 16 * block + orow] = acc[r];
+      }
+    }
+    __syncthreads();
+    if (t0 < N) {
+      const int o = tid, tok = o / EP, e = o - tok * EP;   // RS_THREADS == RR_TOKENS * EP
+      const half_t hv = (half_t)(part[o] + part[RR_TOKENS * EP + o]);
+      lg[o] = hv;
+      if (t0 + tok < N && e < E) logits[(size_t)(t0 + tok) * E + e] = hv;
+    }
+    __syncthreads();
+    // ---- route: one wavefront per token
+    {
+      const int tok = wave, t = t0 + tok;
+      int my_e = -1;
+      if (t < N) {
+        float my_w;
+        route_core::route_token<half_t, 1>(lg + tok * EP, E, k, norm, my_e, my_w);
+        if (lane < k) {
+          idx[(size_t)t * k + lane] = my_e;
+          w[(size_t)t * k + lane] = (half_t)my_w;
+        }
+      }
+      if (lane < k) sidx[(g * RR_TOKENS + tok) * k + lane] = my_e;
+    }
+  }
+  if (!hist_out) return;
+  __syncthreads();
+  if (wave == 0) {
+    for (int e = lane; e < E; e += WAVE) hist[e] = 0;
+    count_piece(sidx, 0, groups * RR_TOKENS * k, E, nbits, hist);
+    for (int e = lane; e < E; e += WAVE) hist_out[(size_t)blockIdx.x * E + e] = hist[e];
+  }
+}
+static_assert(RS_THREADS == RR_TOKENS * 64, "one thread per logit of the workgroup");
+static_assert(RS_WAVES == RR_TOKENS, "one wavefront per token routes");
+static_assert(RS_DEPTH % 2 == 0, "pairs of slices never wrap inside the ring");
+
 bool router_route_shape_ok(int N, int H, int E, int k) {
   return N >= 1 && H >= 512 && H % 512 == 0 && E >= 1 && E <= 128 && k >= 1 && k <= FRONT_MAX_K && k <= E &&
          (long)N * H * 2 < (1l << 31);
@@ -193,6 +348,15 @@ int launch_router_route(const void* h, const void* router, int N, int H, int E, 
   if (hist) {   // one workgroup per piece of the sort, and as many pieces as its second launch reads
     groups = piece_for(M) / (RR_TOKENS * k);
     grid = large_blocks(M) * SORT_WAVES;
+  }
+  if (E <= 64 && H / RS_BK >= RS_DEPTH) {   // staged through LDS (H is a multiple of 512: at least 1024 here)
+    const size_t lds = (size_t)RS_DEPTH * RS_STAGE + sizeof(float) * 2 * RR_TOKENS * 64 + sizeof(half_t) * RR_TOKENS * 64 +
+                       sizeof(int) * ((size_t)groups * RR_TOKENS * k + E);
+    if (hipFuncSetAttribute((const void*)router_route_staged_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return sy_fail(SY_ERR_LAUNCH, "router_route: cannot reserve %zu bytes of LDS", lds);
+    router_route_staged_kernel<<<grid, RS_THREADS, lds, st>>>((const half_t*)h, (const half_t*)router, N, H, E, k, norm, nbits,
+                                                             groups, (half_t*)logits, idx, (half_t*)w, (int*)hist);
+    return sy_check_launch("router_route");
   }
   const int EP = E <= 64 ? 64 : 128;
   const bool wide = E <= 64 && H % 2048 == 0;   // 16 wavefronts: four K steps each at H = 2048
