@@ -1,3 +1,8 @@
+// The front of the layer in fewer launches. Two entry points:
+//   sy_route_sort    a decode step's route and sort in one launch (below);
+//   sy_router_route  for more tokens, the router GEMM and route in one launch, which inside
+//                    sy_moe_experts is also the first pass of the sort (further down).
+//
 // route_sort: route and sort of a decode step in one launch.
 //
 // At a handful of tokens each step is a few microseconds of launch and memory latency around
