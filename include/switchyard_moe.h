@@ -132,7 +132,9 @@ SY_API int sy_combine(const void* y, const int32_t* pos_of, const int32_t* idx, 
  * h f16 [N,H]; router f16 [E,H] or NULL; logits f16 [N,E]; gate_up f16 [E,2I,H]; down f16
  * [E,H,I]; mfma_tiles 0 runs sy_grouped_gemv twice, nonzero sy_grouped_gemm. Outputs as the
  * separate calls' (idx, w, counts, offsets, token, wsorted, pos_of), plus act f16 [N*k, I],
- * y f16 [N*k, H] and out f16 [N,H], all caller-allocated. Limits: those of the entry points it
+ * y f16 [N*k, H] (the down projection's rows BEFORE the router weight: this call applies the
+ * weight in its combine, with the roundings of the separate calls, so `out` has their bits) and
+ * out f16 [N,H], all caller-allocated. Limits: those of the entry points it
  * calls. */
 SY_API int sy_moe_experts(const void* h, const void* router, void* logits, int N, int E, int k, int norm,
                           const void* gate_up, const void* down, int H, int I, int mfma_tiles, int one_launch_front,

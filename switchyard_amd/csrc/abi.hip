@@ -82,15 +82,19 @@ extern "C" SY_API int sy_moe_experts(const void* h, const void* router, void* lo
   }
   if (rc) return rc;
   const int M = N * k;
+  // The down projection runs without its row scales: y holds its rows before the router weight,
+  // and the combine multiplies, with the same roundings in the same order. Fetching the scales
+  // costs the projection's epilogue more than the multiply costs the combine, which waits for
+  // memory either way.
   if (mfma_tiles) {
     rc = sy_grouped_gemm(h, token, gate_up, offsets, E, M, I, H, 1, nullptr, act, stream);
     if (rc) return rc;
-    rc = sy_grouped_gemm(act, nullptr, down, offsets, E, M, H, I, 0, wsorted, y, stream);
+    rc = sy_grouped_gemm(act, nullptr, down, offsets, E, M, H, I, 0, nullptr, y, stream);
   } else {
     rc = sy_grouped_gemv(h, token, gate_up, offsets, E, M, N, I, H, 1, nullptr, act, stream);
     if (rc) return rc;
-    rc = sy_grouped_gemv(act, nullptr, down, offsets, E, M, N, H, I, 0, wsorted, y, stream);
+    rc = sy_grouped_gemv(act, nullptr, down, offsets, E, M, N, H, I, 0, nullptr, y, stream);
   }
   if (rc) return rc;
-  return sy_combine(y, pos_of, idx, N, k, H, out, stream);
+  return sy_combine_weighted(y, pos_of, idx, w, N, k, H, out, stream);
 }

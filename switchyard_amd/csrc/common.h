@@ -31,6 +31,9 @@ int sy_sort_assign_counted(const int32_t* idx, const void* w, int N, int k, int 
 int sy_router_route_counting(const void* h, const void* router, int N, int H, int E, int k, int norm, void* logits,
                              int32_t* idx, void* w, void* hist, void* stream);
 bool sy_router_route_counts(int N, int k);
+// combine.hip: combine of rows that were left unscaled, times the router weights w [N, k]
+int sy_combine_weighted(const void* y, const int32_t* pos_of, const int32_t* idx, const void* w, int N, int k, int H, void* out,
+                        void* stream);
 
 #define SY_REQUIRE(cond, ...) \
   do {                        \
