@@ -49,6 +49,19 @@ SY_API int sy_add_rmsnorm_logits(const void* x, const void* delta, const void* w
  * rows, not thousands (the library GEMM takes over there). Limits: as sy_add_rmsnorm_logits. */
 SY_API int sy_router_logits(const void* h, const void* router, int N, int H, int E, void* logits, void* stream);
 
+/* sy_router_logits, sy_route and sy_sort_by_expert in ONE launch, for a decode step: replaces
+ * `F.linear(h, router)` + route() + sort_by_expert() (switchyard/kernels.py:30-32,84;
+ * switchyard/csrc/moe_kernels.cu:73-89,142-157). One workgroup per token computes its logits as
+ * sy_router_logits does, routes it, and the workgroup that finishes last sorts every token's
+ * choices; outputs (logits included) are bit for bit those of the three separate calls.
+ * Limits: those of sy_router_logits, 1 <= N <= 256, E <= 128, 1 <= k <= min(8, E). N == 0 is a
+ * no-op. The launch counts its workgroups in a counter of a pool of 1024 that the library keeps
+ * in device memory; launches take the counters in turn, so launches on DIFFERENT streams may
+ * only disturb each other if one is still waiting to run when the 1024th after it is issued. */
+SY_API int sy_router_route_sort(const void* h, const void* router, int N, int H, int E, int k, int norm, void* logits,
+                                int32_t* idx, void* w, int32_t* counts, int32_t* offsets, int32_t* token, void* wsorted,
+                                int32_t* pos_of, void* stream);
+
 /* sy_combine folded into the residual add and the next RMS norm: replaces combine()
  * (switchyard/csrc/moe_kernels.cu:435-444) followed by `x = x + moe(i, h)` and the rmsnorm of
  * the next block (switchyard/model.py:142,119 or :130).

@@ -123,9 +123,9 @@ SY_API int sy_combine(const void* y, const int32_t* pos_of, const int32_t* idx, 
 
 /* Replaces moe_layer() (switchyard/kernels.py:91-93: route() with its router GEMM, :30-32, then
  * experts(), :76-88: sort -> pick -> ffn -> combine) in ONE call: the router's logits
- * (when `router` is given: sy_router_logits up to 64 tokens, above that sy_router_route, which
- * routes in the same launch and is also the first pass of the sort; with router NULL `logits` is
- * an input), route and sort (sy_route_sort when one_launch_front is nonzero, else sy_route and
+ * (when `router` is given: up to 64 tokens sy_router_route_sort, which is the whole front in one
+ * launch; above that sy_router_route, which routes in the same launch and is also the first pass
+ * of the sort; with router NULL `logits` is an input), route and sort (sy_route_sort when one_launch_front is nonzero, else sy_route and
  * sy_sort_by_expert with the given workspace), the gate/up projection (SwiGLU, rows of h gathered through `token`), the
  * down projection (x router weight) and sy_combine are enqueued back to back, exactly as the
  * separate calls would be.
@@ -141,6 +141,16 @@ SY_API int sy_moe_experts(const void* h, const void* router, void* logits, int N
                           int32_t* idx, void* w, int32_t* counts, int32_t* offsets, int32_t* token, void* wsorted,
                           int32_t* pos_of, void* act, void* y, void* out, void* sort_workspace,
                           size_t sort_workspace_bytes, void* stream);
+
+/* The part of sy_moe_experts behind the sort, for a caller that has enqueued the front of the
+ * layer on the same stream itself (sy_router_route_sort, or sy_route and sy_sort_by_expert):
+ * replaces pick() / ffn() / combine() as experts() calls them (switchyard/kernels.py:85-88).
+ * Inputs idx int32 [N,k], w f16 [N,k], offsets int32 [E+1], token int32 [N*k], pos_of int32
+ * [N*k] as the front leaves them; act, y (rows before the router weight) and out as in
+ * sy_moe_experts. */
+SY_API int sy_experts_sorted(const void* h, int N, int E, int k, const void* gate_up, const void* down, int H, int I,
+                             int mfma_tiles, const int32_t* idx, const void* w, const int32_t* offsets,
+                             const int32_t* token, const int32_t* pos_of, void* act, void* y, void* out, void* stream);
 
 #ifdef __cplusplus
 }

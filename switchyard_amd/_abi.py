@@ -40,6 +40,9 @@ SIGNATURES = {
     "sy_moe_experts": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p,
                                 _c_int, _c_int, _c_int, _c_int] + [_c_void_p] * 11 + [_c_size_t, _c_void_p]),
     "sy_router_logits": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p]),
+    "sy_router_route_sort": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int] + [_c_void_p] * 9),
+    "sy_experts_sorted": (_c_int, [_c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int]
+                          + [_c_void_p] * 9),
     "sy_router_route": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p,
                                  _c_void_p, _c_void_p]),
     "sy_add_rmsnorm": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_int, _c_int, _c_void_p, _c_void_p,
@@ -222,32 +225,34 @@ class Ext:
         h [N, H] and either logits [N, E] f16 or router [E, H] f16 (then logits is None and the
         library's own router kernel computes them: for tens of tokens) -> out [N, H]. The
         intermediate results live in one scratch allocation and are not returned."""
+        # Only what the front of the layer reads is checked here: a call that is waited for is
+        # timed with the host time in front of its first launch, so the weights of the experts
+        # are checked behind that launch (_enqueue_experts), before anything reads them.
         _check(h, "h", torch.float16)
-        _check(gate_up, "gate_up", torch.float16)
-        _check(down, "down", torch.float16)
         N, H = h.shape
-        E, I = gate_up.shape[0], down.shape[2]
         if (logits is None) == (router is None):
             raise RuntimeError("moe_experts: give the logits or the router")
         if logits is not None:
             _check(logits, "logits", torch.float16)
-            if tuple(logits.shape) != (N, E):
+            E = logits.shape[1]
+            if logits.shape[0] != N:
                 raise RuntimeError("moe_experts: logits must be [N, E]")
         else:
             _check(router, "router", torch.float16)
-            if tuple(router.shape) != (E, H):
+            E = router.shape[0]
+            if router.shape[1] != H:
                 raise RuntimeError("moe_experts: router must be [E, H]")
-        if tuple(gate_up.shape) != (E, 2 * I, H) or tuple(down.shape) != (E, H, I):
-            raise RuntimeError("moe_experts: shapes of h / gate_up / down do not match")
+        if down.dim() != 3:
+            raise RuntimeError("moe_experts: down must be [E, H, I]")
+        I, k, norm = down.shape[2], int(k), int(bool(norm))
         stream = _stream()
         # The intermediate results of small calls (a decode step's) live in an allocation that is
-        # kept per shape and stream: calls on one stream run in order, so they may share it, and a
-        # call once waited for is timed with this function's host time in front of its first launch.
-        key = (N, E, int(k), H, I, logits is None, bool(one_launch_front), h.device.index, stream)
+        # kept per shape and stream: calls on one stream run in order, so they may share it.
+        key = (N, E, k, H, I, norm, logits is None, bool(one_launch_front), h.device.index, stream)
         plan = self._plans.get(key)
         if plan is None:
-            M = N * int(k)
-            need = 0 if one_launch_front else self.lib.sy_sort_workspace_bytes(N, int(k), E)
+            M = N * k
+            need = 0 if one_launch_front else self.lib.sy_sort_workspace_bytes(N, k, E)
             # idx w counts offsets token wsorted pos_of act y, then the sort's workspace and the logits
             sizes = [M * 4, M * 2, E * 4, (E + 1) * 4, M * 4, M * 2, M * 4, M * I * 2, M * H * 2, need,
                      N * E * 2 if logits is None else 0]
@@ -255,42 +260,57 @@ class Ext:
             for size in sizes:
                 starts.append(at)
                 at += (size + 255) // 256 * 256
-            plan = (starts, at, need, None)
+            plan = (starts, at, need, None, None)
             if at <= self.PLAN_BYTES_MAX:
                 if len(self._plans) >= self.PLANS_MAX:
                     self._plans.pop(next(iter(self._plans)))
-                plan = (starts, at, need, torch.empty(at, dtype=torch.uint8, device=h.device))
+                scratch = torch.empty(at, dtype=torch.uint8, device=h.device)
+                plan = (starts, at, need, scratch, self._addresses(scratch, starts))
                 self._plans[key] = plan
-        starts, at, need, scratch = plan
+        starts, at, need, scratch, where = plan
         if scratch is None:
             scratch = torch.empty(at, dtype=torch.uint8, device=h.device)
-            return self._enqueue_experts(h, router, logits, gate_up, down, k, norm, mfma_tiles, one_launch_front,
-                                         scratch, starts, need, stream)
+            return self._enqueue_experts(h, router, logits, gate_up, down, N, H, E, I, k, norm, mfma_tiles, one_launch_front,
+                                         scratch, self._addresses(scratch, starts), need, stream)
         # kept scratch: two threads enqueueing the same shape on one stream must not interleave
         # their launches (ctypes releases the GIL inside the calls)
         with self._plans_lock:
-            return self._enqueue_experts(h, router, logits, gate_up, down, k, norm, mfma_tiles, one_launch_front,
-                                         scratch, starts, need, stream)
+            return self._enqueue_experts(h, router, logits, gate_up, down, N, H, E, I, k, norm, mfma_tiles, one_launch_front,
+                                         scratch, where, need, stream)
 
-    def _enqueue_experts(self, h, router, logits, gate_up, down, k, norm, mfma_tiles, one_launch_front, scratch, starts,
-                         need, stream):
-        N, H = h.shape
-        E, I = gate_up.shape[0], down.shape[2]
+    @staticmethod
+    def _addresses(scratch, starts):
         base = scratch.data_ptr()
+        return tuple(base + s for s in starts)
+
+    def _enqueue_experts(self, h, router, logits, gate_up, down, N, H, E, I, k, norm, mfma_tiles, one_launch_front, scratch,
+                         where, need, stream):
+        lib = self.lib
+        front_done = router is not None and N <= 64 and E <= 128 and 1 <= k <= 8 and k <= E
+        if front_done:
+            # the front of the layer (logits, route and sort: one launch) is enqueued at once: the
+            # GPU works on it while the host checks the weights, allocates the result and
+            # marshals the long call (a call that is waited for starts its first kernel sooner;
+            # in a stream of calls nothing changes)
+            if lib.sy_router_route_sort(h.data_ptr(), router.data_ptr(), N, H, E, k, norm, where[10], *where[:7], stream):
+                raise RuntimeError(lib.sy_last_error().decode())
+        _check(gate_up, "gate_up", torch.float16)
+        _check(down, "down", torch.float16)
+        if tuple(gate_up.shape) != (E, 2 * I, H) or tuple(down.shape) != (E, H, I):
+            raise RuntimeError("moe_experts: shapes of h / gate_up / down do not match")
+        out = torch.empty((N, H), dtype=torch.float16, device=h.device)
+        if front_done:
+            self._call(lib.sy_experts_sorted, h.data_ptr(), N, E, k, gate_up.data_ptr(), down.data_ptr(), H, I,
+                       int(bool(mfma_tiles)), where[0], where[1], where[3], where[4], where[6], where[7], where[8],
+                       out.data_ptr(), stream)
+            return out
         router_ptr = router.data_ptr() if router is not None else None
         if router is not None and N <= 64:
-            # the router's logits are enqueued at once: the GPU works on them while the host
-            # allocates the result and marshals the long call (a call that is waited for starts
-            # its first kernel 4 us sooner; in a stream of calls nothing changes)
-            self._call(self.lib.sy_router_logits, h.data_ptr(), router_ptr, N, H, E, base + starts[10], stream)
+            self._call(lib.sy_router_logits, h.data_ptr(), router_ptr, N, H, E, where[10], stream)
             router_ptr = None
-        out = torch.empty((N, H), dtype=torch.float16, device=h.device)
-        self._call(self.lib.sy_moe_experts, h.data_ptr(), router_ptr,
-                   logits.data_ptr() if logits is not None else base + starts[10], N, E, int(k), int(bool(norm)),
-                   gate_up.data_ptr(), down.data_ptr(), H, I, int(bool(mfma_tiles)), int(bool(one_launch_front)),
-                   base + starts[0], base + starts[1], base + starts[2], base + starts[3], base + starts[4], base + starts[5],
-                   base + starts[6], base + starts[7], base + starts[8], out.data_ptr(), base + starts[9] if need else None,
-                   need, stream)
+        self._call(lib.sy_moe_experts, h.data_ptr(), router_ptr, logits.data_ptr() if logits is not None else where[10],
+                   N, E, k, norm, gate_up.data_ptr(), down.data_ptr(), H, I, int(bool(mfma_tiles)),
+                   int(bool(one_launch_front)), *where[:9], out.data_ptr(), where[9] if need else None, need, stream)
         return out
 
     @staticmethod
@@ -313,6 +333,27 @@ class Ext:
         self._call(self.lib.sy_router_route, h.data_ptr(), router.data_ptr(), N, H, E, int(k), int(bool(norm)),
                    logits.data_ptr(), idx.data_ptr(), w.data_ptr(), _stream())
         return idx, w, logits
+
+    def router_route_sort(self, h, router, k, norm):
+        """h [N, H], router [E, H] -> [logits f16 [N, E], idx [N, k], w [N, k], counts [E], offsets
+        [E+1], token [M], wsorted [M], pos_of [M]]: router_logits, route and sort_by_expert in one
+        launch, for a decode step (at most 256 tokens, 128 experts, top-8)."""
+        _check(h, "h", torch.float16)
+        _check(router, "router", torch.float16)
+        N, H = h.shape
+        E, k = router.shape[0], int(k)
+        if router.shape[1] != H:
+            raise RuntimeError("router_route_sort: h and router must have the same width")
+        dev, M = h.device, N * k
+        i32 = dict(dtype=torch.int32, device=dev)
+        f16 = dict(dtype=torch.float16, device=dev)
+        logits, idx, w = torch.empty((N, E), **f16), torch.empty((N, k), **i32), torch.empty((N, k), **f16)
+        counts, offsets = torch.empty(E, **i32), torch.empty(E + 1, **i32)
+        token, wsorted, pos_of = torch.empty(M, **i32), torch.empty(M, **f16), torch.empty(M, **i32)
+        self._call(self.lib.sy_router_route_sort, h.data_ptr(), router.data_ptr(), N, H, E, k, int(bool(norm)),
+                   logits.data_ptr(), idx.data_ptr(), w.data_ptr(), counts.data_ptr(), offsets.data_ptr(),
+                   token.data_ptr(), wsorted.data_ptr(), pos_of.data_ptr(), _stream())
+        return [logits, idx, w, counts, offsets, token, wsorted, pos_of]
 
     def router_logits(self, h, router):
         """h [N, H] @ router [E, H]^T -> logits [N, E] f16 by the library's own kernel (tens of rows)."""

@@ -66,6 +66,9 @@ extern "C" SY_API int sy_moe_experts(const void* h, const void* router, void* lo
     rc = counted ? sy_sort_assign_counted(idx, w, N, k, E, counts, offsets, token, wsorted, pos_of, sort_workspace, stream)
                  : sy_sort_by_expert(idx, w, 2, N, k, E, counts, offsets, token, wsorted, pos_of, sort_workspace,
                                      sort_workspace_bytes, stream);
+  } else if (router && E <= 128 && k >= 1 && k <= 8 && k <= E) {
+    // a decode step: logits, route and sort in one launch
+    rc = sy_router_route_sort(h, router, N, H, E, k, norm, logits, idx, w, counts, offsets, token, wsorted, pos_of, stream);
   } else {
     if (router) {   // the router GEMM too: logits is then an output
       rc = sy_router_logits(h, router, N, H, E, logits, stream);
@@ -81,6 +84,20 @@ extern "C" SY_API int sy_moe_experts(const void* h, const void* router, void* lo
     }
   }
   if (rc) return rc;
+  return sy_experts_sorted(h, N, E, k, gate_up, down, H, I, mfma_tiles, idx, w, offsets, token, pos_of, act, y, out, stream);
+}
+
+// What follows the sort in sy_moe_experts, for a caller that has enqueued the front itself.
+extern "C" SY_API int sy_experts_sorted(const void* h, int N, int E, int k, const void* gate_up, const void* down, int H, int I,
+                                        int mfma_tiles, const int32_t* idx, const void* w, const int32_t* offsets,
+                                        const int32_t* token, const int32_t* pos_of, void* act, void* y, void* out,
+                                        void* stream) {
+  SY_REQUIRE(N >= 0 && H >= 8 && I >= 8, "experts_sorted: N = %d, H = %d, I = %d", N, H, I);
+  if (N == 0) return SY_OK;
+  SY_REQUIRE(h && act && y && out, "experts_sorted: null pointer");
+  // the projections address the gathered rows of h with 32-bit byte offsets
+  SY_REQUIRE((long)N * H * 2 < (1l << 31), "experts_sorted: h must stay under 2 GiB (%d rows of %d)", N, H);
+  int rc;
   const int M = N * k;
   // The down projection runs without its row scales: y holds its rows before the router weight,
   // and the combine multiplies, with the same roundings in the same order. Fetching the scales

@@ -26,7 +26,10 @@
 // taken in fp32, rounded to fp16 and then scaled in fp16; rotary products and their sum are
 // each rounded to fp16. Attention scores and the softmax stay in fp32 (the reference rounds
 // the scores to fp16 first), which is the more exact of the two.
+#include <mutex>
+
 #include "common.h"
+#include "front_core.h"
 #include "../../include/switchyard_decode.h"
 
 namespace {
@@ -55,13 +58,17 @@ constexpr int ROW_MAX_K = 64;  // choices per token the combining variant ranks 
 // router needs no launch of its own; that variant runs 16 wavefronts, each with the loads of
 // four experts in flight at once, because the router's rows come from L2 one round trip at a
 // time and the trips, not the bytes, are what it waits for.
-template <bool COMBINE, bool LOGITS>
+// With FRONT (and LOGITS) the workgroup then routes its token from the logits in LDS, and the last
+// workgroup of the launch to get there sorts every token's choices (front_core.h): the layer's
+// router GEMM, route and sort in one launch.
+template <bool COMBINE, bool LOGITS, bool FRONT = false>
 __global__ void __launch_bounds__(LOGITS ? 1024 : ROW_THREADS)
 row_kernel(const half_t* x, const half_t* __restrict__ delta, const half_t* __restrict__ y,
            const int* __restrict__ pos_of, const int* __restrict__ idx, int k, const half_t* __restrict__ weight,
            float eps, const half_t* __restrict__ router, int E, int H, half_t* x_out, half_t* __restrict__ h_out,
-           half_t* __restrict__ logits, const int64_t* __restrict__ gather, int src_rows) {  // x_out may be x
-  extern __shared__ __attribute__((aligned(16))) half_t hs[];  // LOGITS: the normalised row [H]
+           half_t* __restrict__ logits, const int64_t* __restrict__ gather, int src_rows,
+           front_core::Outputs front = front_core::Outputs{}) {  // x_out may be x
+  extern __shared__ __attribute__((aligned(16))) half_t hs[];  // LOGITS: the normalised row [H]; FRONT: the tail's LDS behind it
   __shared__ float part[16];
   __shared__ int rows[ROW_MAX_K];
   const int t = blockIdx.x, tid = threadIdx.x, nthreads = blockDim.x;
@@ -179,8 +186,19 @@ row_kernel(const half_t* x, const half_t* __restrict__ delta, const half_t* __re
     for (int u = 0; u < 4; ++u) {
       const float total = wave_sum(acc[u]);
       const int e = e0 + nwaves * u;
-      if (lane == 0 && e < E) logits[(size_t)t * E + e] = (half_t)total;
+      if (lane == 0 && e < E) {
+        logits[(size_t)t * E + e] = (half_t)total;
+        if (FRONT) hs[H + e] = (half_t)total;
+      }
     }
+  }
+  if (FRONT) {
+    __syncthreads();
+    unsigned char* tail = reinterpret_cast<unsigned char*>(hs + H);
+    if (E <= 64)
+      front_core::route_own_sort_last<1>(t, (int)gridDim.x, E, front, tail);
+    else
+      front_core::route_own_sort_last<2>(t, (int)gridDim.x, E, front, tail);
   }
 }
 
@@ -669,6 +687,68 @@ extern "C" SY_API int sy_router_logits(const void* h, const void* router, int N,
       (const half_t*)h, nullptr, nullptr, nullptr, nullptr, 0, nullptr, 0.f, (const half_t*)router, E, H, nullptr, nullptr,
       (half_t*)logits, nullptr, 0);
   return sy_check_launch("router_logits");
+}
+
+// The counters of the launches that end in front_core's tail. Every GPU the library runs on
+// holds its own copy, all zero when the module is loaded and again after every launch. In host
+// code the array's name is only a handle for hipGetSymbolAddress: launches take next_ticket()'s
+// pointer.
+static __device__ unsigned front_tickets[front_core::FRONT_TICKETS];
+
+namespace {
+constexpr int TICKET_DEVICES = 64;
+std::mutex ticket_mutex;
+unsigned* ticket_base[TICKET_DEVICES] = {nullptr};
+unsigned ticket_next[TICKET_DEVICES] = {0};
+
+// The counter for the next launch on the current device: slots are handed out in turn.
+int next_ticket(unsigned** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= TICKET_DEVICES)
+    return sy_fail(SY_ERR_LAUNCH, "router_route_sort: no current device below %d", TICKET_DEVICES);
+  std::lock_guard<std::mutex> hold(ticket_mutex);
+  if (!ticket_base[dev]) {
+    void* p = nullptr;
+    const hipError_t err = hipGetSymbolAddress(&p, HIP_SYMBOL(front_tickets));
+    if (err != hipSuccess || !p)
+      return sy_fail(SY_ERR_LAUNCH, "router_route_sort: hipGetSymbolAddress: %s", hipGetErrorString(err));
+    ticket_base[dev] = static_cast<unsigned*>(p);
+  }
+  *out = ticket_base[dev] + ticket_next[dev]++ % front_core::FRONT_TICKETS;
+  return SY_OK;
+}
+
+int front_outputs(const char* what, int N, int E, int k, int norm, int32_t* idx, void* w, int32_t* counts, int32_t* offsets,
+                  int32_t* token, void* wsorted, int32_t* pos_of, front_core::Outputs* out) {
+  SY_REQUIRE(N <= front_core::TAIL_MAX_TOKENS, "%s: at most %d tokens (got %d)", what, front_core::TAIL_MAX_TOKENS, N);
+  SY_REQUIRE(E <= 128 && k >= 1 && k <= front_core::TAIL_MAX_K && k <= E, "%s: at most 128 experts and top-8 (got E = %d, k = %d)",
+             what, E, k);
+  SY_REQUIRE(idx && w && counts && offsets && token && wsorted && pos_of, "%s: null pointer", what);
+  unsigned* ticket = nullptr;
+  const int rc = next_ticket(&ticket);
+  if (rc) return rc;
+  int nbits = 0;
+  while ((1 << nbits) < E) ++nbits;
+  *out = front_core::Outputs{idx, (half_t*)w, counts, offsets, token, (half_t*)wsorted, pos_of, ticket, k, norm, nbits};
+  return SY_OK;
+}
+}  // namespace
+
+extern "C" SY_API int sy_router_route_sort(const void* h, const void* router, int N, int H, int E, int k, int norm, void* logits,
+                                           int32_t* idx, void* w, int32_t* counts, int32_t* offsets, int32_t* token,
+                                           void* wsorted, int32_t* pos_of, void* stream) {
+  ROW_LIMITS("router_route_sort");
+  SY_REQUIRE(E >= 1, "router_route_sort: E = %d", E);
+  if (N == 0) return SY_OK;
+  SY_REQUIRE(h && router && logits, "router_route_sort: null pointer");
+  front_core::Outputs front;
+  const int rc = front_outputs("router_route_sort", N, E, k, norm, idx, w, counts, offsets, token, wsorted, pos_of, &front);
+  if (rc) return rc;
+  const size_t lds = (size_t)H * sizeof(half_t) + front_core::tail_lds_bytes(N, E, k);
+  row_kernel<false, true, true><<<N, 1024, lds, (hipStream_t)stream>>>(
+      (const half_t*)h, nullptr, nullptr, nullptr, nullptr, 0, nullptr, 0.f, (const half_t*)router, E, H, nullptr, nullptr,
+      (half_t*)logits, nullptr, 0, front);
+  return sy_check_launch("router_route_sort");
 }
 
 extern "C" SY_API int sy_combine_add_rmsnorm(const void* y, const int32_t* pos_of, const int32_t* idx, int k, const void* x,

@@ -27,10 +27,11 @@ def declared_symbols(header=None):
 def test_header_declares_the_expected_entry_points():
     assert sorted(declared_symbols(DECODE_HEADER)) == ["sy_add_rmsnorm", "sy_add_rmsnorm_logits", "sy_combine_add_rmsnorm",
                                                        "sy_decode_attention", "sy_decode_attention_qkv", "sy_embed_rmsnorm",
-                                                       "sy_greedy_advance", "sy_qk_norm_rope_cache", "sy_router_logits"]
+                                                       "sy_greedy_advance", "sy_qk_norm_rope_cache", "sy_router_logits",
+                                                           "sy_router_route_sort"]
     assert sorted(os.listdir(os.path.join(ROOT, "include"))) == ["switchyard_decode.h", "switchyard_moe.h"]
     assert sorted(declared_symbols(HEADER)) == sorted(["sy_version", "sy_last_error", "sy_route", "sy_sort_workspace_bytes",
-                                                  "sy_sort_by_expert", "sy_sort_by_expert_static", "sy_route_sort", "sy_router_route",
+                                                  "sy_sort_by_expert", "sy_sort_by_expert_static", "sy_route_sort", "sy_router_route", "sy_experts_sorted",
                                                   "sy_grouped_gemv", "sy_grouped_gemm",
                                                   "sy_combine", "sy_moe_experts"])
 

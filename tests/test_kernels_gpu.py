@@ -433,6 +433,69 @@ def test_route_sort_in_one_launch(K, N, E, k, H, norm):
     assert torch.equal(wsorted.cpu().view(torch.int16), p.weight.view(torch.int16))
 
 
+@pytest.mark.parametrize("N,E,k,H", [(1, 64, 8, 2048), (8, 64, 8, 2048), (9, 64, 8, 2048), (16, 64, 8, 2048),
+                                     (64, 64, 8, 2048), (256, 64, 8, 256), (7, 128, 8, 512), (20, 16, 3, 128),
+                                     (5, 60, 3, 64), (64, 64, 1, 256), (33, 100, 5, 1024)])
+@pytest.mark.parametrize("norm", [False, True])
+def test_router_logits_route_and_sort_in_one_launch(K, N, E, k, H, norm):
+    """Bit for bit what router_logits, route and sort_by_expert give in three launches, and the
+    oracle's route and plan on those logits; called three times in a row, because every launch
+    must leave its counter as it found it."""
+    g = torch.Generator().manual_seed(N * 11 + E)
+    h = torch.randn(N, H, generator=g).half().to(DEV)
+    router = (torch.randn(E, H, generator=g) * H ** -0.5).half().to(DEV)
+    ext = K.ext()
+    rlogits = ext.router_logits(h, router)
+    ridx, rw = ext.route(rlogits, k, norm)
+    rsort = ext.sort_by_expert(ridx, rw, E)
+    for _ in range(3):
+        logits, idx, w, *sort = ext.router_route_sort(h, router, k, norm)
+        assert torch.equal(logits, rlogits)
+        assert torch.equal(idx, ridx) and torch.equal(w, rw)
+        for a, b in zip(sort, rsort):
+            assert torch.equal(a, b)
+    oidx, ow = O.route_logits(logits.cpu(), k, norm)
+    assert torch.equal(idx.cpu().long(), oidx)
+    p = O.plan(oidx, w.cpu(), E)
+    counts, offsets, token, wsorted, pos_of = sort
+    assert torch.equal(counts.cpu().long(), p.counts) and torch.equal(offsets.cpu().long(), p.offsets)
+    assert torch.equal(token.cpu().long(), p.token) and torch.equal(pos_of.cpu().long(), p.pos_of)
+    assert torch.equal(wsorted.cpu().view(torch.int16), p.weight.view(torch.int16))
+
+
+def test_router_route_sort_counters_come_round(K):
+    """More launches than the library keeps counters, of two sizes in turn: a launch that finds a
+    counter not at zero would sort too early or never."""
+    g = torch.Generator().manual_seed(5)
+    ext = K.ext()
+    cases = []
+    for N in (8, 13):
+        h = torch.randn(N, 512, generator=g).half().to(DEV)
+        router = (torch.randn(64, 512, generator=g) * 512 ** -0.5).half().to(DEV)
+        logits = ext.router_logits(h, router)
+        idx, w = ext.route(logits, 8, False)
+        cases.append((h, router, ext.sort_by_expert(idx, w, 64)))
+    results = []
+    for i in range(1100):
+        h, router, _ = cases[i % 2]
+        results.append(ext.router_route_sort(h, router, 8, False)[3:])
+    torch.cuda.synchronize()
+    for i, got in enumerate(results):
+        for a, b in zip(got, cases[i % 2][2]):
+            assert torch.equal(a, b), i
+
+
+def test_router_route_sort_limits(K):
+    h = torch.zeros(4, 256, dtype=torch.float16, device=DEV)
+    with pytest.raises(RuntimeError):
+        K.ext().router_route_sort(torch.zeros(300, 256, dtype=torch.float16, device=DEV),
+                                  torch.zeros(64, 256, dtype=torch.float16, device=DEV), 8, False)   # too many tokens
+    with pytest.raises(RuntimeError):
+        K.ext().router_route_sort(h, torch.zeros(64, 256, dtype=torch.float16, device=DEV), 9, False)
+    with pytest.raises(RuntimeError):
+        K.ext().router_route_sort(h, torch.zeros(200, 256, dtype=torch.float16, device=DEV), 8, False)  # too many experts
+
+
 def test_route_sort_limits(K):
     with pytest.raises(RuntimeError):
         K.ext().route_sort(torch.zeros(300, 64, dtype=torch.float16, device=DEV), 8, False)   # too many tokens
