@@ -43,6 +43,17 @@ SY_API int sy_embed_rmsnorm(const int64_t* tokens, const void* embed, int vocab,
 SY_API int sy_add_rmsnorm_logits(const void* x, const void* delta, const void* weight, float eps, const void* router,
                                  int E, int N, int H, void* x_out, void* h_out, void* logits, void* stream);
 
+/* sy_add_rmsnorm_logits with the front of the MoE layer in the same launch: every token's
+ * workgroup also routes it, and the last one to finish sorts (as sy_router_route_sort below,
+ * whose limits and note on the launch counter apply): replaces the residual add, the RMS norm,
+ * the router GEMM, route() and sort_by_expert() of a decode step (switchyard/model.py:119-121,
+ * switchyard/kernels.py:30-32,84). Outputs are bit for bit those of sy_add_rmsnorm_logits
+ * followed by sy_route and sy_sort_by_expert. */
+SY_API int sy_add_rmsnorm_route_sort(const void* x, const void* delta, const void* weight, float eps, const void* router,
+                                     int E, int N, int H, int k, int norm, void* x_out, void* h_out, void* logits,
+                                     int32_t* idx, void* w, int32_t* counts, int32_t* offsets, int32_t* token,
+                                     void* wsorted, int32_t* pos_of, void* stream);
+
 /* The router GEMM alone, for a few rows (a decode step): replaces `F.linear(h, router)`
  * (switchyard/kernels.py:30-32). h f16 [N,H]; router f16 [E,H] -> logits f16 [N,E], fp32 sums
  * rounded once. One workgroup per row reads the whole router from L2, so this is for tens of
@@ -67,9 +78,14 @@ SY_API int sy_router_route_sort(const void* h, const void* router, int N, int H,
  * the next block (switchyard/model.py:142,119 or :130).
  * y f16 [M,H], pos_of int32 [N*k], idx int32 [N,k] as sy_combine takes them; x f16 [N,H] ->
  * x_out = f16(x + d) with d the f16 result sy_combine would give (the same bits), and
- * h_out = the RMS norm of x_out as sy_add_rmsnorm. Limits: as sy_add_rmsnorm, 1 <= k <= 64. */
-SY_API int sy_combine_add_rmsnorm(const void* y, const int32_t* pos_of, const int32_t* idx, int k, const void* x,
-                                  const void* weight, float eps, int N, int H, void* x_out, void* h_out, void* stream);
+ * h_out = the RMS norm of x_out as sy_add_rmsnorm. w is NULL, or the router weights f16 [N,k]
+ * (route's output) when y holds the down projection's rows BEFORE the router weight (scale NULL
+ * in sy_grouped_gemv / sy_grouped_gemm): each row is then multiplied and rounded to f16 here as
+ * the projection's epilogue would have, so the results have the same bits either way, and the
+ * projection does not fetch a scale per row. Limits: as sy_add_rmsnorm, 1 <= k <= 64. */
+SY_API int sy_combine_add_rmsnorm(const void* y, const int32_t* pos_of, const int32_t* idx, const void* w, int k,
+                                  const void* x, const void* weight, float eps, int N, int H, void* x_out, void* h_out,
+                                  void* stream);
 
 /* What follows the q/k/v projections of T new tokens per sequence (T = 1 at decode, the prompt
  * length at prefill); replaces the rmsnorm of q and k, the clamp, the rotary embedding and the

@@ -53,7 +53,9 @@ SIGNATURES = {
                                    _c_void_p, _c_void_p]),
     "sy_add_rmsnorm_logits": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_int, _c_int,
                                        _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
-    "sy_combine_add_rmsnorm": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_float, _c_int,
+    "sy_add_rmsnorm_route_sort": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_int, _c_int,
+                                           _c_int, _c_int] + [_c_void_p] * 11),
+    "sy_combine_add_rmsnorm": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_float, _c_int,
                                         _c_int, _c_void_p, _c_void_p, _c_void_p]),
     "sy_qk_norm_rope_cache": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_float, _c_void_p, _c_void_p, _c_int,
                                        _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p,
@@ -367,10 +369,12 @@ class Ext:
         return logits
 
     # ---- the decode-step kernels around the MoE layer (include/switchyard_decode.h)
-    def add_rmsnorm(self, x, delta, weight, eps, x_out=None, router=None):
+    def add_rmsnorm(self, x, delta, weight, eps, x_out=None, router=None, front=None):
         """x [N, H] (+ delta [N, H] or None) -> (x + delta, weight * rmsnorm(x + delta)).
         With delta None the first result is x itself; x_out may be x for an update in place.
-        With `router` [E, H] a third result is the logits [N, E] of the normalised rows."""
+        With `router` [E, H] a third result is the logits [N, E] of the normalised rows; with
+        front = (top_k, norm_topk_prob) as well (at most 256 rows, 128 experts, top-8) the launch
+        also routes and sorts, and route_sort's seven results follow the logits."""
         _check(x, "x", torch.float16)
         _check(weight, "weight", torch.float16)
         N, H = x.shape
@@ -397,6 +401,19 @@ class Ext:
         if router.dim() != 2 or router.shape[1] != H:
             raise RuntimeError("add_rmsnorm: router must be [E, H]")
         logits = torch.empty((N, router.shape[0]), dtype=torch.float16, device=x.device)
+        if front is not None:
+            E, k, dev = router.shape[0], int(front[0]), x.device
+            M = N * k
+            i32 = dict(dtype=torch.int32, device=dev)
+            idx, w = torch.empty((N, k), **i32), torch.empty((N, k), dtype=torch.float16, device=dev)
+            counts, offsets = torch.empty(E, **i32), torch.empty(E + 1, **i32)
+            token, pos_of = torch.empty(M, **i32), torch.empty(M, **i32)
+            wsorted = torch.empty(M, dtype=torch.float16, device=dev)
+            self._call(self.lib.sy_add_rmsnorm_route_sort, x.data_ptr(), d_ptr, weight.data_ptr(), float(eps),
+                       router.data_ptr(), E, N, H, k, int(bool(front[1])), o_ptr, h.data_ptr(), logits.data_ptr(),
+                       idx.data_ptr(), w.data_ptr(), counts.data_ptr(), offsets.data_ptr(), token.data_ptr(),
+                       wsorted.data_ptr(), pos_of.data_ptr(), _stream())
+            return first, h, logits, idx, w, counts, offsets, token, wsorted, pos_of
         self._call(self.lib.sy_add_rmsnorm_logits, x.data_ptr(), d_ptr, weight.data_ptr(), float(eps), router.data_ptr(),
                    router.shape[0], N, H, o_ptr, h.data_ptr(), logits.data_ptr(), _stream())
         return first, h, logits
@@ -429,9 +446,11 @@ class Ext:
         self._call(self.lib.sy_greedy_advance, logits.data_ptr(), B, V, tok.data_ptr(), out.data_ptr(), out.shape[1],
                    base_position.data_ptr(), next_position.data_ptr(), slot.data_ptr(), _stream())
 
-    def combine_add_rmsnorm(self, y, pos_of, idx, x, weight, eps, x_out=None):
+    def combine_add_rmsnorm(self, y, pos_of, idx, x, weight, eps, x_out=None, w=None):
         """combine(y, pos_of, idx) added to x [N, H] and normalised in one launch ->
-        (x + combine, weight * rmsnorm(x + combine)); x_out may be x."""
+        (x + combine, weight * rmsnorm(x + combine)); x_out may be x. With w [N, k] (route's
+        weights) y holds the down projection's rows before the router weight, which is applied
+        here: the same bits as rows scaled where they were computed."""
         _check(y, "y", torch.float16)
         _check(pos_of, "pos_of", torch.int32)
         _check(idx, "idx", torch.int32)
@@ -445,7 +464,12 @@ class Ext:
             x_out = torch.empty_like(x)
         _check(x_out, "x_out", torch.float16)
         h = torch.empty_like(x)
-        self._call(self.lib.sy_combine_add_rmsnorm, y.data_ptr(), pos_of.data_ptr(), idx.data_ptr(), k, x.data_ptr(),
+        if w is not None:
+            _check(w, "w", torch.float16)
+            if w.numel() < N * k:
+                raise RuntimeError("combine_add_rmsnorm: w shorter than N * k")
+        self._call(self.lib.sy_combine_add_rmsnorm, y.data_ptr(), pos_of.data_ptr(), idx.data_ptr(),
+                   w.data_ptr() if w is not None else None, k, x.data_ptr(),
                    weight.data_ptr(), float(eps), N, H, x_out.data_ptr(), h.data_ptr(), _stream())
         return x_out, h
 

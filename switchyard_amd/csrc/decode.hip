@@ -52,7 +52,8 @@ constexpr int ROW_MAX_K = 64;  // choices per token the combining variant ranks 
 
 // One workgroup per token (row). The residual `delta` is either a tensor, or (COMBINE) the
 // token's k expert outputs summed in fp32 in ascending expert id and rounded to f16 once,
-// exactly as the combine kernel leaves it; then x_out = f16(x + delta) and h = the RMS norm
+// exactly as the combine kernel leaves it (`delta` then holds the router weights [N, k] of rows
+// that the down projection left unscaled, or is null); then x_out = f16(x + delta) and h = the RMS norm
 // of x_out. With LOGITS the normalised row stays in LDS and the four wavefronts also take its
 // dot products with the E rows of the router (fp32 sums, one rounding to f16), so that the
 // router needs no launch of its own; that variant runs 16 wavefronts, each with the loads of
@@ -71,6 +72,7 @@ row_kernel(const half_t* x, const half_t* __restrict__ delta, const half_t* __re
   extern __shared__ __attribute__((aligned(16))) half_t hs[];  // LOGITS: the normalised row [H]; FRONT: the tail's LDS behind it
   __shared__ float part[16];
   __shared__ int rows[ROW_MAX_K];
+  __shared__ float wts[ROW_MAX_K];   // COMBINE: the router weight of each row, 1 where y is already scaled
   const int t = blockIdx.x, tid = threadIdx.x, nthreads = blockDim.x;
   const size_t row = (size_t)t * H;
   const int chunks = H >> 3;
@@ -91,7 +93,10 @@ row_kernel(const half_t* x, const half_t* __restrict__ delta, const half_t* __re
         const int other = read_lane(mine, j);
         rank += (other < mine) || (other == mine && j < tid);
       }
-      if (tid < k) rows[rank] = src;
+      if (tid < k) {
+        rows[rank] = src;
+        wts[rank] = delta ? (float)delta[(size_t)t * k + tid] : 1.f;
+      }
     }
     __syncthreads();
   }
@@ -106,8 +111,10 @@ row_kernel(const half_t* x, const half_t* __restrict__ delta, const half_t* __re
         float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         for (int j = 0; j < k; ++j) {
           const half8_t e = *reinterpret_cast<const half8_t*>(y + (size_t)rows[j] * H + c * 8);
+          const float wt = wts[j];
+          // the rounding of the down projection's scaled epilogue (times 1 it changes nothing)
 #pragma unroll
-          for (int q = 0; q < 8; ++q) acc[q] += (float)e[q];
+          for (int q = 0; q < 8; ++q) acc[q] += (float)(half_t)((float)e[q] * wt);
         }
 #pragma unroll
         for (int q = 0; q < 8; ++q) v[i][q] = (half_t)((float)v[i][q] + (float)(half_t)acc[q]);
@@ -751,15 +758,34 @@ extern "C" SY_API int sy_router_route_sort(const void* h, const void* router, in
   return sy_check_launch("router_route_sort");
 }
 
-extern "C" SY_API int sy_combine_add_rmsnorm(const void* y, const int32_t* pos_of, const int32_t* idx, int k, const void* x,
-                                             const void* weight, float eps, int N, int H, void* x_out, void* h_out,
-                                             void* stream) {
+extern "C" SY_API int sy_add_rmsnorm_route_sort(const void* x, const void* delta, const void* weight, float eps,
+                                                const void* router, int E, int N, int H, int k, int norm, void* x_out,
+                                                void* h_out, void* logits, int32_t* idx, void* w, int32_t* counts,
+                                                int32_t* offsets, int32_t* token, void* wsorted, int32_t* pos_of,
+                                                void* stream) {
+  ROW_LIMITS("add_rmsnorm_route_sort");
+  SY_REQUIRE(E >= 1, "add_rmsnorm_route_sort: E = %d", E);
+  if (N == 0) return SY_OK;
+  SY_REQUIRE(x && weight && h_out && router && logits, "add_rmsnorm_route_sort: null pointer");
+  front_core::Outputs front;
+  const int rc = front_outputs("add_rmsnorm_route_sort", N, E, k, norm, idx, w, counts, offsets, token, wsorted, pos_of, &front);
+  if (rc) return rc;
+  const size_t lds = (size_t)H * sizeof(half_t) + front_core::tail_lds_bytes(N, E, k);
+  row_kernel<false, true, true><<<N, 1024, lds, (hipStream_t)stream>>>(
+      (const half_t*)x, (const half_t*)delta, nullptr, nullptr, nullptr, 0, (const half_t*)weight, eps,
+      (const half_t*)router, E, H, (half_t*)x_out, (half_t*)h_out, (half_t*)logits, nullptr, 0, front);
+  return sy_check_launch("add_rmsnorm_route_sort");
+}
+
+extern "C" SY_API int sy_combine_add_rmsnorm(const void* y, const int32_t* pos_of, const int32_t* idx, const void* w, int k,
+                                             const void* x, const void* weight, float eps, int N, int H, void* x_out,
+                                             void* h_out, void* stream) {
   ROW_LIMITS("combine_add_rmsnorm");
   SY_REQUIRE(k >= 1 && k <= ROW_MAX_K, "combine_add_rmsnorm: 1 <= k <= %d (got %d)", ROW_MAX_K, k);
   if (N == 0) return SY_OK;
   SY_REQUIRE(y && pos_of && idx && x && weight && h_out, "combine_add_rmsnorm: null pointer");
   row_kernel<true, false><<<N, ROW_THREADS, 0, (hipStream_t)stream>>>(
-      (const half_t*)x, nullptr, (const half_t*)y, pos_of, idx, k, (const half_t*)weight, eps, nullptr, 0, H,
+      (const half_t*)x, (const half_t*)w, (const half_t*)y, pos_of, idx, k, (const half_t*)weight, eps, nullptr, 0, H,
       (half_t*)x_out, (half_t*)h_out, nullptr, nullptr, 0);
   return sy_check_launch("combine_add_rmsnorm");
 }

@@ -358,9 +358,19 @@ class Decoder:
             o = kernels.dense(a, L["wo"])
             if self._own_moe and s.experts <= 1024 and s.top_k <= 64:
                 # the router's logits come out of the norm's launch, and combine goes into the next norm's
-                x, h, logits = E.add_rmsnorm(x, o, L["mlp_norm"], s.rms_eps, x_out=x, router=L["router"])
-                y, pos_of, idx = kernels.experts_rows(h, logits, L["gate_up"], L["down"], s.top_k, s.norm_topk_prob)
-                x, xn = E.combine_add_rmsnorm(y, pos_of, idx, x, after, s.rms_eps, x_out=x)
+                if x.shape[0] <= 256 and s.experts <= 128 and s.top_k <= min(8, s.experts):
+                    # ... and so do route and sort
+                    # ... and so do route and sort; the router weights are applied where the rows
+                    # are combined (the down projection then fetches no scale per row)
+                    x, h, _, idx, w, counts, offsets, token, _, pos_of = E.add_rmsnorm(
+                        x, o, L["mlp_norm"], s.rms_eps, x_out=x, router=L["router"], front=(s.top_k, s.norm_topk_prob))
+                    y = kernels.ffn(h, token, offsets, counts, None, L["gate_up"], L["down"], idx.numel(),
+                                    kernels._auto(x.shape[0], idx.numel(), s.experts))
+                else:
+                    x, h, logits = E.add_rmsnorm(x, o, L["mlp_norm"], s.rms_eps, x_out=x, router=L["router"])
+                    y, pos_of, idx = kernels.experts_rows(h, logits, L["gate_up"], L["down"], s.top_k, s.norm_topk_prob)
+                    w = None
+                x, xn = E.combine_add_rmsnorm(y, pos_of, idx, x, after, s.rms_eps, x_out=x, w=w)
             else:
                 x, h = E.add_rmsnorm(x, o, L["mlp_norm"], s.rms_eps, x_out=x)
                 x, xn = E.add_rmsnorm(x, self.moe(i, h), after, s.rms_eps, x_out=x)

@@ -25,7 +25,8 @@ def declared_symbols(header=None):
 
 
 def test_header_declares_the_expected_entry_points():
-    assert sorted(declared_symbols(DECODE_HEADER)) == ["sy_add_rmsnorm", "sy_add_rmsnorm_logits", "sy_combine_add_rmsnorm",
+    assert sorted(declared_symbols(DECODE_HEADER)) == ["sy_add_rmsnorm", "sy_add_rmsnorm_logits", "sy_add_rmsnorm_route_sort",
+                                                           "sy_combine_add_rmsnorm",
                                                        "sy_decode_attention", "sy_decode_attention_qkv", "sy_embed_rmsnorm",
                                                        "sy_greedy_advance", "sy_qk_norm_rope_cache", "sy_router_logits",
                                                            "sy_router_route_sort"]
@@ -71,9 +72,15 @@ def test_decode_argument_errors_and_empty_batches(lib):
     assert lib.sy_greedy_advance(None, 4, 1000, None, None, 8, None, None, None, None) == 1   # null pointers
     assert lib.sy_add_rmsnorm_logits(None, None, None, 1e-5, None, 2000, 4, 2048, None, None, None, None) == 1
     assert lib.sy_add_rmsnorm_logits(None, None, None, 1e-5, None, 64, 0, 2048, None, None, None, None) == 0
-    assert lib.sy_combine_add_rmsnorm(None, None, None, 65, None, None, 1e-5, 4, 2048, None, None, None) == 1
-    assert lib.sy_combine_add_rmsnorm(None, None, None, 8, None, None, 1e-5, 4, 2044, None, None, None) == 1
-    assert lib.sy_combine_add_rmsnorm(None, None, None, 8, None, None, 1e-5, 0, 2048, None, None, None) == 0
+    assert lib.sy_combine_add_rmsnorm(None, None, None, None, 65, None, None, 1e-5, 4, 2048, None, None, None) == 1
+    assert lib.sy_combine_add_rmsnorm(None, None, None, None, 8, None, None, 1e-5, 4, 2044, None, None, None) == 1
+    assert lib.sy_combine_add_rmsnorm(None, None, None, None, 8, None, None, 1e-5, 0, 2048, None, None, None) == 0
+    nine = (None,) * 9
+    assert lib.sy_router_route_sort(None, None, 0, 2048, 64, 8, 0, *nine) == 0
+    assert lib.sy_router_route_sort(None, None, 4, 2044, 64, 8, 0, *nine) == 1
+    assert lib.sy_router_route_sort(None, None, 4, 2048, 64, 8, 0, *nine) == 1          # null pointers
+    assert lib.sy_add_rmsnorm_route_sort(None, None, None, 1e-5, None, 64, 0, 2048, 8, 0, *nine, None, None) == 0
+    assert lib.sy_add_rmsnorm_route_sort(None, None, None, 1e-5, None, 64, 4, 2048, 8, 0, *nine, None, None) == 1
     assert lib.sy_qk_norm_rope_cache(None, None, None, 1e-5, 0.0, None, None, 64, None, None, 2, 1, 16, 5, 128, 64, None,
                                      None, None, None) == 1
     assert lib.sy_qk_norm_rope_cache(None, None, None, 1e-5, 0.0, None, None, 64, None, None, 2, 1, 16, 16, 72, 64, None,

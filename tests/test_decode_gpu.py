@@ -59,6 +59,29 @@ def test_add_rmsnorm_with_router_logits(N, H, E):
     assert torch.allclose(logits3.float(), h3.float() @ router.float().T, rtol=ULP, atol=1e-4)
 
 
+@pytest.mark.parametrize("N,H,E,k", [(8, 2048, 64, 8), (64, 2048, 64, 8), (3, 512, 16, 4), (13, 520, 7, 3), (256, 256, 128, 8)])
+@pytest.mark.parametrize("norm", [False, True])
+def test_add_rmsnorm_with_logits_route_and_sort(N, H, E, k, norm):
+    """The launch that also routes and sorts gives the bits of add_rmsnorm with the router,
+    route and sort_by_expert in three launches; twice, so that the second finds the launch
+    counter as the first left it."""
+    x, d, w = rnd(N, H, seed=1), rnd(N, H, seed=2, std=0.3), 1 + rnd(H, seed=3, std=0.1)
+    router = rnd(E, H, seed=4, std=0.02)
+    ext = kernels.ext()
+    xo, h, logits = ext.add_rmsnorm(x, d, w, 1e-5, router=router)
+    idx, wts = ext.route(logits, k, norm)
+    want = [xo, h, logits, idx, wts] + list(ext.sort_by_expert(idx, wts, E))
+    for delta in (d, d, None):
+        got = ext.add_rmsnorm(x, delta, w, 1e-5, router=router, front=(k, norm))
+        if delta is None:
+            _, h0, logits0 = ext.add_rmsnorm(x, None, w, 1e-5, router=router)
+            idx0, w0 = ext.route(logits0, k, norm)
+            want = [x, h0, logits0, idx0, w0] + list(ext.sort_by_expert(idx0, w0, E))
+        assert len(got) == len(want) == 10
+        for a, b in zip(got, want):
+            assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("N,H,E,k", [(8, 2048, 64, 8), (64, 2048, 64, 8), (5, 512, 16, 4), (1, 64, 8, 2), (300, 256, 64, 8)])
 def test_combine_add_rmsnorm(N, H, E, k):
     """combine, residual add and norm in one launch give the bits of the three launches."""
@@ -72,6 +95,11 @@ def test_combine_add_rmsnorm(N, H, E, k):
     xo, h = ext.add_rmsnorm(x, delta, w, 1e-5)
     xo2, h2 = ext.combine_add_rmsnorm(y, pos_of, idx, x, w, 1e-5)
     assert torch.equal(xo2, xo) and torch.equal(h2, h)
+    # rows not yet scaled, the router weights applied in the same launch: the bits of scaling first
+    scaled = (y.float() * wsorted.float()[:, None]).half()
+    xo3, h3 = ext.combine_add_rmsnorm(scaled, pos_of, idx, x, w, 1e-5)
+    xo4, h4 = ext.combine_add_rmsnorm(y, pos_of, idx, x, w, 1e-5, w=wts)
+    assert torch.equal(xo4, xo3) and torch.equal(h4, h3)
     x3 = x.clone()
     xo3, h3 = ext.combine_add_rmsnorm(y, pos_of, idx, x3, w, 1e-5, x_out=x3)
     assert xo3 is x3 and torch.equal(x3, xo) and torch.equal(h3, h)
