@@ -132,8 +132,9 @@ SY_API int sy_combine(const void* y, const int32_t* pos_of, const int32_t* idx, 
  * h f16 [N,H]; router f16 [E,H] or NULL; logits f16 [N,E]; gate_up f16 [E,2I,H]; down f16
  * [E,H,I]; mfma_tiles 0 runs sy_grouped_gemv twice, nonzero sy_grouped_gemm. Outputs as the
  * separate calls' (idx, w, counts, offsets, token, wsorted, pos_of), plus act f16 [N*k, I],
- * y f16 [N*k, H] (the down projection's rows BEFORE the router weight: this call applies the
- * weight in its combine, with the roundings of the separate calls, so `out` has their bits) and
+ * y f16 [N*k, H] (scratch: the down projection's rows, before or after the router weight; with
+ * the weight-stream kernels and with the 256-row MFMA tile this call applies the weight in its
+ * combine instead, with the roundings of the separate calls, so `out` has their bits) and
  * out f16 [N,H], all caller-allocated. Limits: those of the entry points it
  * calls. */
 SY_API int sy_moe_experts(const void* h, const void* router, void* logits, int N, int E, int k, int norm,
@@ -145,12 +146,12 @@ SY_API int sy_moe_experts(const void* h, const void* router, void* logits, int N
 /* The part of sy_moe_experts behind the sort, for a caller that has enqueued the front of the
  * layer on the same stream itself (sy_router_route_sort, or sy_route and sy_sort_by_expert):
  * replaces pick() / ffn() / combine() as experts() calls them (switchyard/kernels.py:85-88).
- * Inputs idx int32 [N,k], w f16 [N,k], offsets int32 [E+1], token int32 [N*k], pos_of int32
- * [N*k] as the front leaves them; act, y (rows before the router weight) and out as in
- * sy_moe_experts. */
+ * Inputs idx int32 [N,k], w f16 [N,k], offsets int32 [E+1], token int32 [N*k], wsorted f16
+ * [N*k], pos_of int32 [N*k] as the front leaves them; act, y and out as in sy_moe_experts. */
 SY_API int sy_experts_sorted(const void* h, int N, int E, int k, const void* gate_up, const void* down, int H, int I,
                              int mfma_tiles, const int32_t* idx, const void* w, const int32_t* offsets,
-                             const int32_t* token, const int32_t* pos_of, void* act, void* y, void* out, void* stream);
+                             const int32_t* token, const void* wsorted, const int32_t* pos_of, void* act, void* y,
+                             void* out, void* stream);
 
 #ifdef __cplusplus
 }

@@ -42,7 +42,7 @@ SIGNATURES = {
     "sy_router_logits": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p]),
     "sy_router_route_sort": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int] + [_c_void_p] * 9),
     "sy_experts_sorted": (_c_int, [_c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int]
-                          + [_c_void_p] * 9),
+                          + [_c_void_p] * 10),
     "sy_router_route": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p,
                                  _c_void_p, _c_void_p]),
     "sy_add_rmsnorm": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_int, _c_int, _c_void_p, _c_void_p,
@@ -303,7 +303,7 @@ class Ext:
         out = torch.empty((N, H), dtype=torch.float16, device=h.device)
         if front_done:
             self._call(lib.sy_experts_sorted, h.data_ptr(), N, E, k, gate_up.data_ptr(), down.data_ptr(), H, I,
-                       int(bool(mfma_tiles)), where[0], where[1], where[3], where[4], where[6], where[7], where[8],
+                       int(bool(mfma_tiles)), where[0], where[1], where[3], where[4], where[5], where[6], where[7], where[8],
                        out.data_ptr(), stream)
             return out
         router_ptr = router.data_ptr() if router is not None else None

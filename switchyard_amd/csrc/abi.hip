@@ -84,14 +84,15 @@ extern "C" SY_API int sy_moe_experts(const void* h, const void* router, void* lo
     }
   }
   if (rc) return rc;
-  return sy_experts_sorted(h, N, E, k, gate_up, down, H, I, mfma_tiles, idx, w, offsets, token, pos_of, act, y, out, stream);
+  return sy_experts_sorted(h, N, E, k, gate_up, down, H, I, mfma_tiles, idx, w, offsets, token, wsorted, pos_of, act, y, out,
+                           stream);
 }
 
 // What follows the sort in sy_moe_experts, for a caller that has enqueued the front itself.
 extern "C" SY_API int sy_experts_sorted(const void* h, int N, int E, int k, const void* gate_up, const void* down, int H, int I,
                                         int mfma_tiles, const int32_t* idx, const void* w, const int32_t* offsets,
-                                        const int32_t* token, const int32_t* pos_of, void* act, void* y, void* out,
-                                        void* stream) {
+                                        const int32_t* token, const void* wsorted, const int32_t* pos_of, void* act,
+                                        void* y, void* out, void* stream) {
   SY_REQUIRE(N >= 0 && H >= 8 && I >= 8, "experts_sorted: N = %d, H = %d, I = %d", N, H, I);
   if (N == 0) return SY_OK;
   SY_REQUIRE(h && act && y && out, "experts_sorted: null pointer");
@@ -99,19 +100,24 @@ extern "C" SY_API int sy_experts_sorted(const void* h, int N, int E, int k, cons
   SY_REQUIRE((long)N * H * 2 < (1l << 31), "experts_sorted: h must stay under 2 GiB (%d rows of %d)", N, H);
   int rc;
   const int M = N * k;
-  // The down projection runs without its row scales: y holds its rows before the router weight,
-  // and the combine multiplies, with the same roundings in the same order. Fetching the scales
-  // costs the projection's epilogue more than the multiply costs the combine, which waits for
-  // memory either way.
+  // Where it pays, the down projection runs without its row scales: y then holds its rows before
+  // the router weight, and the combine multiplies, with the same roundings in the same order.
+  // Fetching the scales costs the weight-stream kernel and the 256-row MFMA tile (which the
+  // GEMM picks from about 108 rows per expert on) more than the multiply costs the combine
+  // (8 tokens: 0.7 us against 0.1; 4096: 3 to 9 us against 0.7); the smaller MFMA tiles gain
+  // nothing, so there the projection scales. `out` has the same bits either way.
+  const bool combine_scales = !mfma_tiles || (long)M >= 108l * E;
+  const void* scale = combine_scales ? nullptr : wsorted;
   if (mfma_tiles) {
     rc = sy_grouped_gemm(h, token, gate_up, offsets, E, M, I, H, 1, nullptr, act, stream);
     if (rc) return rc;
-    rc = sy_grouped_gemm(act, nullptr, down, offsets, E, M, H, I, 0, nullptr, y, stream);
+    rc = sy_grouped_gemm(act, nullptr, down, offsets, E, M, H, I, 0, scale, y, stream);
   } else {
     rc = sy_grouped_gemv(h, token, gate_up, offsets, E, M, N, I, H, 1, nullptr, act, stream);
     if (rc) return rc;
-    rc = sy_grouped_gemv(act, nullptr, down, offsets, E, M, N, H, I, 0, nullptr, y, stream);
+    rc = sy_grouped_gemv(act, nullptr, down, offsets, E, M, N, H, I, 0, scale, y, stream);
   }
   if (rc) return rc;
-  return sy_combine_weighted(y, pos_of, idx, w, N, k, H, out, stream);
+  return combine_scales ? sy_combine_weighted(y, pos_of, idx, w, N, k, H, out, stream)
+                        : sy_combine(y, pos_of, idx, N, k, H, out, stream);
 }
