@@ -95,8 +95,8 @@ def _auto(n_tokens, n_choices, n_experts):
 
 def ffn(x, a_rows, offsets, counts, wsorted, gate_up, down, rows, mode, host_counts=None):
     """Both projections of the experts for `rows` sorted rows -> y [rows, H], router weight
-    already applied (wsorted None: not applied, for a combine that multiplies). offsets [E + 1] cuts the sorted rows into one run per expert; sorted row i
-    reads x[a_rows[i]] (x[i] if a_rows is None), so the unsorted activations are never copied.
+    already applied (wsorted None: not applied, for a combine that multiplies). offsets [E + 1]
+    cuts the sorted rows into one run per expert; sorted row i reads x[a_rows[i]] (x[i] if a_rows is None), so the unsorted activations are never copied.
     mode is "gemv" or "gemm" ("cublas" means "gemm" here). `counts` and `host_counts` only keep
     the reference's argument list (kernels.py:48): no launch here depends on a value read
     back from the GPU."""

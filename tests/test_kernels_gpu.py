@@ -485,6 +485,31 @@ def test_router_route_sort_counters_come_round(K):
             assert torch.equal(a, b), i
 
 
+def test_router_route_sort_on_two_streams_at_once(K):
+    """Launches on different streams take different counters, so they may run side by side."""
+    g = torch.Generator().manual_seed(9)
+    ext = K.ext()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    cases = []
+    for N in (8, 40):
+        h = torch.randn(N, 2048, generator=g).half().to(DEV)
+        router = (torch.randn(64, 2048, generator=g) * 2048 ** -0.5).half().to(DEV)
+        logits = ext.router_logits(h, router)
+        idx, w = ext.route(logits, 8, True)
+        cases.append((h, router, [logits, idx, w] + list(ext.sort_by_expert(idx, w, 64))))
+    torch.cuda.synchronize()
+    results = ([], [])
+    for _ in range(60):
+        for s in (0, 1):
+            with torch.cuda.stream(streams[s]):
+                results[s].append(ext.router_route_sort(cases[s][0], cases[s][1], 8, True))
+    torch.cuda.synchronize()
+    for s in (0, 1):
+        for got in results[s]:
+            for a, b in zip(got, cases[s][2]):
+                assert torch.equal(a, b)
+
+
 def test_router_route_sort_limits(K):
     h = torch.zeros(4, 256, dtype=torch.float16, device=DEV)
     with pytest.raises(RuntimeError):
