@@ -68,7 +68,9 @@ SY_API int sy_router_logits(const void* h, const void* router, int N, int H, int
  * Limits: those of sy_router_logits, 1 <= N <= 256, E <= 128, 1 <= k <= min(8, E). N == 0 is a
  * no-op. The launch counts its workgroups in a counter of a pool of 1024 that the library keeps
  * in device memory; launches take the counters in turn, so launches on DIFFERENT streams may
- * only disturb each other if one is still waiting to run when the 1024th after it is issued. */
+ * only disturb each other if one is still waiting to run when the 1024th after it is issued.
+ * The first call on a device looks the pool's address up (hipGetSymbolAddress): make one call
+ * outside stream capture before capturing one. */
 SY_API int sy_router_route_sort(const void* h, const void* router, int N, int H, int E, int k, int norm, void* logits,
                                 int32_t* idx, void* w, int32_t* counts, int32_t* offsets, int32_t* token, void* wsorted,
                                 int32_t* pos_of, void* stream);
