@@ -611,3 +611,31 @@ def test_experts_in_one_call_equal_the_five_calls(K, N, E, k, H, I, tiles, norm)
     if N <= K.OWN_ROUTER_MAX_TOKENS or fused_router:     # and with the router GEMM inside the same call
         assert torch.equal(ext.moe_experts(h, None, gu, dn, k, norm, mfma_tiles=tiles, one_launch_front=one_launch,
                                            router=router), want)
+
+
+@pytest.mark.parametrize("N,tiles", [(1, False), (8, False), (40, True), (64, True)])
+def test_moe_experts_entry_point_with_a_router_at_decode_sizes(K, N, tiles):
+    """The C entry point itself, called as a foreign binding would (one call, the router given):
+    up to 64 tokens it runs the one-launch front, which the Python binding enqueues separately."""
+    E, k, H, I = 64, 8, 512, 128
+    h, router, gu, dn = (t.to(DEV) for t in cases.layer(N, E=E, k=k, H=H, I=I, seed=4, wstd=0.05))
+    ext = K.ext()
+    want = K.moe_layer(h, router, gu, dn, k, True, mode="gemm" if tiles else "gemv")
+    M = N * k
+    i32 = dict(dtype=torch.int32, device=DEV)
+    f16 = dict(dtype=torch.float16, device=DEV)
+    logits, idx, w = torch.empty(N, E, **f16), torch.empty(N, k, **i32), torch.empty(N, k, **f16)
+    counts, offsets = torch.empty(E, **i32), torch.empty(E + 1, **i32)
+    token, wsorted, pos_of = torch.empty(M, **i32), torch.empty(M, **f16), torch.empty(M, **i32)
+    act, y, out = torch.empty(M, I, **f16), torch.empty(M, H, **f16), torch.empty(N, H, **f16)
+    rc = ext.lib.sy_moe_experts(h.data_ptr(), router.data_ptr(), logits.data_ptr(), N, E, k, 1, gu.data_ptr(), dn.data_ptr(),
+                                H, I, int(tiles), 0, idx.data_ptr(), w.data_ptr(), counts.data_ptr(), offsets.data_ptr(),
+                                token.data_ptr(), wsorted.data_ptr(), pos_of.data_ptr(), act.data_ptr(), y.data_ptr(),
+                                out.data_ptr(), None, 0, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, ext.lib.sy_last_error()
+    assert torch.equal(out, want)
+    assert torch.equal(logits, ext.router_logits(h, router))
+    ridx, rw = ext.route(logits, k, True)
+    assert torch.equal(idx, ridx) and torch.equal(w, rw)
+    for a, b in zip((counts, offsets, token, wsorted, pos_of), ext.sort_by_expert(ridx, rw, E)):
+        assert torch.equal(a, b)
