@@ -435,7 +435,8 @@ def test_route_sort_in_one_launch(K, N, E, k, H, norm):
 
 @pytest.mark.parametrize("N,E,k,H", [(1, 64, 8, 2048), (8, 64, 8, 2048), (9, 64, 8, 2048), (16, 64, 8, 2048),
                                      (64, 64, 8, 2048), (256, 64, 8, 256), (7, 128, 8, 512), (20, 16, 3, 128),
-                                     (5, 60, 3, 64), (64, 64, 1, 256), (33, 100, 5, 1024)])
+                                     (5, 60, 3, 64), (64, 64, 1, 256), (33, 100, 5, 1024),
+                                     (256, 128, 8, 8192), (12, 64, 8, 2056)])   # the largest shape; a ragged row
 @pytest.mark.parametrize("norm", [False, True])
 def test_router_logits_route_and_sort_in_one_launch(K, N, E, k, H, norm):
     """Bit for bit what router_logits, route and sort_by_expert give in three launches, and the
