@@ -8,8 +8,12 @@
 //
 //   row_kernel            one token per workgroup: x += delta; h = w * f16(x * rsqrt(mean(x^2) + eps)).
 //                         x may be an embedding lookup (embed_rmsnorm), delta may be the combine
-//                         of the MoE layer's rows (combine_add_rmsnorm), and the router's logits
-//                         of h may come out of the same launch (add_rmsnorm_logits)
+//                         of the MoE layer's rows (combine_add_rmsnorm, which also applies
+//                         the router weights to rows that were left unscaled), and the router's
+//                         logits of h may come out of the same launch (add_rmsnorm_logits); with
+//                         them route and the sort as well (add_rmsnorm_route_sort, and
+//                         router_route_sort for rows that need no norm: front_core.h), the whole
+//                         front of the MoE layer in the launch that the step needs anyway
 //   qk_norm_rope_cache    q/k RMS norm over the whole projection, clamp, rotary embedding, and
 //                         the new keys and values written into the cache from `slot` on (one
 //                         token per sequence at decode, the whole prompt at prefill)

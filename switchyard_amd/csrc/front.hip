@@ -2,6 +2,8 @@
 //   sy_route_sort    a decode step's route and sort in one launch (below);
 //   sy_router_route  for more tokens, the router GEMM and route in one launch, which inside
 //                    sy_moe_experts is also the first pass of the sort (further down).
+// (The decode step's router GEMM, route and sort in one launch, sy_router_route_sort, is the
+// row kernel of decode.hip with front_core.h's tail: one workgroup per token, not one in all.)
 //
 // route_sort: route and sort of a decode step in one launch.
 //
