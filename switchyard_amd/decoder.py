@@ -271,8 +271,8 @@ class Decoder:
             o = kernels.dense(a.transpose(1, 2).reshape(B * T, s.heads * s.head_dim), L["wo"])
             x, h = E.add_rmsnorm(x, o, L["mlp_norm"], s.rms_eps, x_out=x)
             if self._own_moe and s.top_k <= 64:
-                logits = F.linear(h, L["router"])
-                y, pos_of, idx = kernels.experts_rows(h, logits, L["gate_up"], L["down"], s.top_k, s.norm_topk_prob)
+                y, pos_of, idx = kernels.experts_rows(h, None, L["gate_up"], L["down"], s.top_k, s.norm_topk_prob,
+                                                      router=L["router"])
                 x, xn = E.combine_add_rmsnorm(y, pos_of, idx, x, after, s.rms_eps, x_out=x)
             else:
                 x, xn = E.add_rmsnorm(x, self.moe(i, h).contiguous(), after, s.rms_eps, x_out=x)

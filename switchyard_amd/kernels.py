@@ -96,10 +96,10 @@ def _auto(n_tokens, n_choices, n_experts):
 def ffn(x, a_rows, offsets, counts, wsorted, gate_up, down, rows, mode, host_counts=None):
     """Both projections of the experts for `rows` sorted rows -> y [rows, H], router weight
     already applied (wsorted None: not applied, for a combine that multiplies). offsets [E + 1]
-    cuts the sorted rows into one run per expert; sorted row i reads x[a_rows[i]] (x[i] if a_rows is None), so the unsorted activations are never copied.
-    mode is "gemv" or "gemm" ("cublas" means "gemm" here). `counts` and `host_counts` only keep
-    the reference's argument list (kernels.py:48): no launch here depends on a value read
-    back from the GPU."""
+    cuts the sorted rows into one run per expert; sorted row i reads x[a_rows[i]] (x[i] if
+    a_rows is None), so the unsorted activations are never copied. mode is "gemv" or "gemm"
+    ("cublas" means "gemm" here). `counts` and `host_counts` only keep the reference's argument
+    list (kernels.py:48): no launch here depends on a value read back from the GPU."""
     E = ext()
     if rows == 0:
         return torch.empty(0, down.shape[1], dtype=x.dtype, device=x.device)
@@ -157,14 +157,18 @@ def dense(x, weight):
 FUSED_FRONT_MAX_TOKENS = 16
 
 
-def experts_rows(h, logits, gate_up, down, top_k, norm_topk_prob, mode="auto"):
+def experts_rows(h, logits, gate_up, down, top_k, norm_topk_prob, mode="auto", router=None):
     """The MoE layer from its router logits [N, E] up to, not including, combine: returns
     (y [N*k, H] expert outputs scaled by the router weights, pos_of, idx), which `combine`
     or a kernel that folds it into what follows takes. Route and sort are one launch up to
-    FUSED_FRONT_MAX_TOKENS tokens."""
+    FUSED_FRONT_MAX_TOKENS tokens. With logits None the router [E, H] is given instead and
+    `route` computes them (for a prompt: the router GEMM and route in one launch)."""
     E = ext()
     N, n_experts = h.shape[0], gate_up.shape[0]
-    if 0 < N <= FUSED_FRONT_MAX_TOKENS and n_experts <= 128 and top_k <= 8 and logits.dtype == torch.float16:
+    if logits is None:
+        idx, w = route(h, router, top_k, norm_topk_prob)
+        counts, offsets, token, wsorted, pos_of = E.sort_by_expert(idx, w, n_experts)
+    elif 0 < N <= FUSED_FRONT_MAX_TOKENS and n_experts <= 128 and top_k <= 8 and logits.dtype == torch.float16:
         idx, w, counts, offsets, token, wsorted, pos_of = E.route_sort(logits, top_k, norm_topk_prob)
     else:
         idx, w = E.route(logits, top_k, norm_topk_prob)
