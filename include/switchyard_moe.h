@@ -75,11 +75,14 @@ SY_API int sy_sort_by_expert_static(const int32_t* idx, const void* w, int w_byt
                                     int32_t* counts, int32_t* offsets, int32_t* token, void* wsorted,
                                     int32_t* pos_of, void* stream);
 
-/* The router GEMM and route() in ONE launch, for more tokens than a decode step has.
+/* The router GEMM and route() in ONE launch.
  * Fuses F.linear(h, router) + route() (switchyard/kernels.py:30-32; kernel moe_kernels.cu:23-71):
  * h f16 [N,H]; router f16 [E,H] -> logits f16 [N,E] (fp32 sums in a fixed order, rounded once),
- * and from those logits exactly the outputs of sy_route (idx, w in f16).
- * Limits: H a multiple of 512, E <= 128, k <= 8, N*H*2 < 2 GiB. N == 0 is a no-op. */
+ * and from those logits exactly the outputs of sy_route (idx, w in f16). Up to 64 tokens a
+ * workgroup per token computes the logits as sy_router_logits does (the same bits) and routes it;
+ * above, 16 tokens to a workgroup on MFMA.
+ * Limits: E <= 128, k <= 8; up to 64 tokens H a multiple of 8 up to 8192, above H a multiple of
+ * 512 and N*H*2 < 2 GiB. N == 0 is a no-op. */
 SY_API int sy_router_route(const void* h, const void* router, int N, int H, int E, int k, int norm, void* logits,
                            int32_t* idx, void* w, void* stream);
 
@@ -124,7 +127,8 @@ SY_API int sy_combine(const void* y, const int32_t* pos_of, const int32_t* idx, 
 /* Replaces moe_layer() (switchyard/kernels.py:91-93: route() with its router GEMM, :30-32, then
  * experts(), :76-88: sort -> pick -> ffn -> combine) in ONE call: the router's logits
  * (when `router` is given: up to 64 tokens sy_router_route_sort, which is the whole front in one
- * launch; above that sy_router_route, which routes in the same launch and is also the first pass
+ * launch, or, with the weight-stream kernels and at most 64 choices, sy_router_route and a
+ * gate/up projection that sorts for itself; above that sy_router_route, which routes in the same launch and is also the first pass
  * of the sort; with router NULL `logits` is an input), route and sort (sy_route_sort when one_launch_front is nonzero, else sy_route and
  * sy_sort_by_expert with the given workspace), the gate/up projection (SwiGLU, rows of h gathered through `token`), the
  * down projection (x router weight) and sy_combine are enqueued back to back, exactly as the
@@ -142,6 +146,18 @@ SY_API int sy_moe_experts(const void* h, const void* router, void* logits, int N
                           int32_t* idx, void* w, int32_t* counts, int32_t* offsets, int32_t* token, void* wsorted,
                           int32_t* pos_of, void* act, void* y, void* out, void* sort_workspace,
                           size_t sort_workspace_bytes, void* stream);
+
+/* Replaces experts() (switchyard/kernels.py:76-88: sort -> pick -> ffn -> combine, for routing
+ * computed elsewhere) in ONE call. idx int32 [N,k] and w f16 [N,k] are inputs; counts ... pos_of
+ * are the sort's outputs as sy_sort_by_expert leaves them, act / y / out as in sy_moe_experts.
+ * With the weight-stream kernels (mfma_tiles 0) and at most 64 choices (N*k <= 64, E <= 128,
+ * H <= 4096) there is no sort launch: the gate/up projection sorts in its own prologue and its
+ * first workgroup writes the sort's outputs; otherwise sy_sort_by_expert runs with the given
+ * workspace (sy_sort_workspace_bytes). `out` has the bits of the separate calls. */
+SY_API int sy_experts_routed(const void* h, int N, int E, int k, const void* gate_up, const void* down, int H, int I,
+                             int mfma_tiles, const int32_t* idx, const void* w, int32_t* counts, int32_t* offsets,
+                             int32_t* token, void* wsorted, int32_t* pos_of, void* act, void* y, void* out,
+                             void* sort_workspace, size_t sort_workspace_bytes, void* stream);
 
 /* The part of sy_moe_experts behind the sort, for a caller that has enqueued the front of the
  * layer on the same stream itself (sy_router_route_sort, or sy_route and sy_sort_by_expert):

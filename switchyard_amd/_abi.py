@@ -43,6 +43,8 @@ SIGNATURES = {
     "sy_router_route_sort": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int] + [_c_void_p] * 9),
     "sy_experts_sorted": (_c_int, [_c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int]
                           + [_c_void_p] * 10),
+    "sy_experts_routed": (_c_int, [_c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int]
+                          + [_c_void_p] * 11 + [_c_size_t, _c_void_p]),
     "sy_router_route": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p,
                                  _c_void_p, _c_void_p]),
     "sy_add_rmsnorm": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_int, _c_int, _c_void_p, _c_void_p,
@@ -280,6 +282,35 @@ class Ext:
             return self._enqueue_experts(h, router, logits, gate_up, down, N, H, E, I, k, norm, mfma_tiles, one_launch_front,
                                          scratch, where, need, stream)
 
+    def experts_routed(self, h, idx, w, gate_up, down, mfma_tiles=False):
+        """experts() of the reference in one call of the library: h [N, H], idx int32 [N, k],
+        w f16 [N, k] -> out [N, H] (sort, the two projections, combine). The intermediate
+        results are allocated here and not returned."""
+        for t, name, dt in ((h, "h", torch.float16), (idx, "idx", torch.int32), (w, "w", torch.float16),
+                            (gate_up, "gate_up", torch.float16), (down, "down", torch.float16)):
+            _check(t, name, dt)
+        N, H = h.shape
+        k, E, I = idx.shape[1], gate_up.shape[0], down.shape[2]
+        if tuple(idx.shape) != (N, k) or tuple(w.shape) != (N, k):
+            raise RuntimeError("experts_routed: idx and w must be [N, k]")
+        if tuple(gate_up.shape) != (E, 2 * I, H) or tuple(down.shape) != (E, H, I):
+            raise RuntimeError("experts_routed: shapes of h / gate_up / down do not match")
+        M = N * k
+        need = self.lib.sy_sort_workspace_bytes(N, k, E)
+        # idx-independent scratch: counts offsets token wsorted pos_of act y, then the sort's workspace
+        sizes = [E * 4, (E + 1) * 4, M * 4, M * 2, M * 4, M * I * 2, M * H * 2, need]
+        starts, at = [], 0
+        for size in sizes:
+            starts.append(at)
+            at += (size + 255) // 256 * 256
+        scratch = torch.empty(max(at, 1), dtype=torch.uint8, device=h.device)
+        where = self._addresses(scratch, starts)
+        out = torch.empty((N, H), dtype=torch.float16, device=h.device)
+        self._call(self.lib.sy_experts_routed, h.data_ptr(), N, E, k, gate_up.data_ptr(), down.data_ptr(), H, I,
+                   int(bool(mfma_tiles)), idx.data_ptr(), w.data_ptr(), *where[:7], out.data_ptr(),
+                   where[7] if need else None, need, _stream())
+        return out
+
     @staticmethod
     def _addresses(scratch, starts):
         base = scratch.data_ptr()
@@ -289,18 +320,31 @@ class Ext:
                          where, need, stream):
         lib = self.lib
         front_done = router is not None and N <= 64 and E <= 128 and 1 <= k <= 8 and k <= E
+        # at most 64 choices on the weight-stream kernels: the front only routes, and the first
+        # projection sorts for itself (sy_experts_routed)
+        routed_only = front_done and not mfma_tiles and N * k <= 64 and H <= 4096
         if front_done:
-            # the front of the layer (logits, route and sort: one launch) is enqueued at once: the
-            # GPU works on it while the host checks the weights, allocates the result and
-            # marshals the long call (a call that is waited for starts its first kernel sooner;
-            # in a stream of calls nothing changes)
-            if lib.sy_router_route_sort(h.data_ptr(), router.data_ptr(), N, H, E, k, norm, where[10], *where[:7], stream):
+            # the front of the layer (logits and route, or logits, route and sort: one launch) is
+            # enqueued at once: the GPU works on it while the host checks the weights, allocates
+            # the result and marshals the long call (a call that is waited for starts its first
+            # kernel sooner; in a stream of calls nothing changes)
+            if routed_only:
+                rc = lib.sy_router_route(h.data_ptr(), router.data_ptr(), N, H, E, k, norm, where[10], where[0], where[1],
+                                         stream)
+            else:
+                rc = lib.sy_router_route_sort(h.data_ptr(), router.data_ptr(), N, H, E, k, norm, where[10], *where[:7],
+                                              stream)
+            if rc:
                 raise RuntimeError(lib.sy_last_error().decode())
         _check(gate_up, "gate_up", torch.float16)
         _check(down, "down", torch.float16)
         if tuple(gate_up.shape) != (E, 2 * I, H) or tuple(down.shape) != (E, H, I):
             raise RuntimeError("moe_experts: shapes of h / gate_up / down do not match")
         out = torch.empty((N, H), dtype=torch.float16, device=h.device)
+        if routed_only:
+            self._call(lib.sy_experts_routed, h.data_ptr(), N, E, k, gate_up.data_ptr(), down.data_ptr(), H, I, 0,
+                       *where[:9], out.data_ptr(), None, 0, stream)
+            return out
         if front_done:
             self._call(lib.sy_experts_sorted, h.data_ptr(), N, E, k, gate_up.data_ptr(), down.data_ptr(), H, I,
                        int(bool(mfma_tiles)), where[0], where[1], where[3], where[4], where[5], where[6], where[7], where[8],

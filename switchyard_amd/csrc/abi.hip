@@ -66,6 +66,13 @@ extern "C" SY_API int sy_moe_experts(const void* h, const void* router, void* lo
     rc = counted ? sy_sort_assign_counted(idx, w, N, k, E, counts, offsets, token, wsorted, pos_of, sort_workspace, stream)
                  : sy_sort_by_expert(idx, w, 2, N, k, E, counts, offsets, token, wsorted, pos_of, sort_workspace,
                                      sort_workspace_bytes, stream);
+  } else if (router && !mfma_tiles && sy_gemv_sorts(N, k, E, H)) {
+    // a decode step of at most 64 choices: logits and route in one launch, and the first
+    // projection sorts for itself
+    rc = sy_router_route_rows(h, router, N, H, E, k, norm, logits, idx, w, stream);
+    if (rc) return rc;
+    return sy_experts_routed(h, N, E, k, gate_up, down, H, I, 0, idx, w, counts, offsets, token, wsorted, pos_of, act, y, out,
+                             sort_workspace, sort_workspace_bytes, stream);
   } else if (router && E <= 128 && k >= 1 && k <= 8 && k <= E) {
     // a decode step: logits, route and sort in one launch
     rc = sy_router_route_sort(h, router, N, H, E, k, norm, logits, idx, w, counts, offsets, token, wsorted, pos_of, stream);
@@ -83,6 +90,30 @@ extern "C" SY_API int sy_moe_experts(const void* h, const void* router, void* lo
                              sort_workspace_bytes, stream);
     }
   }
+  if (rc) return rc;
+  return sy_experts_sorted(h, N, E, k, gate_up, down, H, I, mfma_tiles, idx, w, offsets, token, wsorted, pos_of, act, y, out,
+                           stream);
+}
+
+// experts() of the reference in one call: sort, the two projections, combine, from the routing.
+extern "C" SY_API int sy_experts_routed(const void* h, int N, int E, int k, const void* gate_up, const void* down, int H, int I,
+                                        int mfma_tiles, const int32_t* idx, const void* w, int32_t* counts, int32_t* offsets,
+                                        int32_t* token, void* wsorted, int32_t* pos_of, void* act, void* y, void* out,
+                                        void* sort_workspace, size_t sort_workspace_bytes, void* stream) {
+  SY_REQUIRE(N >= 0 && H >= 8 && I >= 8 && k >= 1, "experts_routed: N = %d, H = %d, I = %d, k = %d", N, H, I, k);
+  if (N == 0) return SY_OK;
+  SY_REQUIRE(h && idx && w && act && y && out, "experts_routed: null pointer");
+  int rc;
+  if (!mfma_tiles && sy_gemv_sorts(N, k, E, H)) {
+    // at most 64 choices: the gate/up stream sorts them in its own prologue
+    rc = sy_grouped_gemv_sorting(h, idx, w, N, k, gate_up, E, I, H, counts, offsets, token, wsorted, pos_of, act, stream);
+    if (rc) return rc;
+    rc = sy_grouped_gemv(act, nullptr, down, offsets, E, N * k, N, H, I, 0, nullptr, y, stream);
+    if (rc) return rc;
+    return sy_combine_weighted(y, pos_of, idx, w, N, k, H, out, stream);
+  }
+  rc = sy_sort_by_expert(idx, w, 2, N, k, E, counts, offsets, token, wsorted, pos_of, sort_workspace, sort_workspace_bytes,
+                         stream);
   if (rc) return rc;
   return sy_experts_sorted(h, N, E, k, gate_up, down, H, I, mfma_tiles, idx, w, offsets, token, wsorted, pos_of, act, y, out,
                            stream);

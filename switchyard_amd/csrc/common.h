@@ -31,6 +31,14 @@ int sy_sort_assign_counted(const int32_t* idx, const void* w, int N, int k, int 
 int sy_router_route_counting(const void* h, const void* router, int N, int H, int E, int k, int norm, void* logits,
                              int32_t* idx, void* w, void* hist, void* stream);
 bool sy_router_route_counts(int N, int k);
+// decode.hip: router GEMM + route for a few rows (one workgroup per row)
+int sy_router_route_rows(const void* h, const void* router, int N, int H, int E, int k, int norm, void* logits, int32_t* idx,
+                         void* w, void* stream);
+// gemv.hip: the gate/up projection of a decode step that sorts its (at most 64) choices itself
+bool sy_gemv_sorts(int N, int k, int E, int H);
+int sy_grouped_gemv_sorting(const void* h, const int32_t* idx, const void* w, int N, int k, const void* gate_up, int E, int I,
+                            int H, int32_t* counts, int32_t* offsets, int32_t* token, void* wsorted, int32_t* pos_of,
+                            void* act, void* stream);
 // combine.hip: combine of rows that were left unscaled, times the router weights w [N, k]
 int sy_combine_weighted(const void* y, const int32_t* pos_of, const int32_t* idx, const void* w, int N, int k, int H, void* out,
                         void* stream);

@@ -63,10 +63,11 @@ constexpr int ROW_MAX_K = 64;  // choices per token the combining variant ranks 
 // router needs no launch of its own; that variant runs 16 wavefronts, each with the loads of
 // four experts in flight at once, because the router's rows come from L2 one round trip at a
 // time and the trips, not the bytes, are what it waits for.
-// With FRONT (and LOGITS) the workgroup then routes its token from the logits in LDS, and the last
-// workgroup of the launch to get there sorts every token's choices (front_core.h): the layer's
-// router GEMM, route and sort in one launch.
-template <bool COMBINE, bool LOGITS, bool FRONT = false>
+// With FRONT (and LOGITS) the workgroup then routes its token from the logits in LDS; with FRONT
+// == FRONT_SORT the last workgroup of the launch to get there also sorts every token's choices
+// (front_core.h): the layer's router GEMM, route and sort in one launch.
+constexpr int FRONT_ROUTE = 1, FRONT_SORT = 2;
+template <bool COMBINE, bool LOGITS, int FRONT = 0>
 __global__ void __launch_bounds__(LOGITS ? 1024 : ROW_THREADS)
 row_kernel(const half_t* x, const half_t* __restrict__ delta, const half_t* __restrict__ y,
            const int* __restrict__ pos_of, const int* __restrict__ idx, int k, const half_t* __restrict__ weight,
@@ -206,10 +207,14 @@ row_kernel(const half_t* x, const half_t* __restrict__ delta, const half_t* __re
   if (FRONT) {
     __syncthreads();
     unsigned char* tail = reinterpret_cast<unsigned char*>(hs + H);
-    if (E <= 64)
+    if (FRONT == FRONT_ROUTE) {
+      if (E <= 64) front_core::route_own<1>(t, E, front, tail);
+      else front_core::route_own<2>(t, E, front, tail);
+    } else if (E <= 64) {
       front_core::route_own_sort_last<1>(t, (int)gridDim.x, E, front, tail);
-    else
+    } else {
       front_core::route_own_sort_last<2>(t, (int)gridDim.x, E, front, tail);
+    }
   }
 }
 
@@ -756,10 +761,27 @@ extern "C" SY_API int sy_router_route_sort(const void* h, const void* router, in
   const int rc = front_outputs("router_route_sort", N, E, k, norm, idx, w, counts, offsets, token, wsorted, pos_of, &front);
   if (rc) return rc;
   const size_t lds = (size_t)H * sizeof(half_t) + front_core::tail_lds_bytes(N, E, k);
-  row_kernel<false, true, true><<<N, 1024, lds, (hipStream_t)stream>>>(
+  row_kernel<false, true, FRONT_SORT><<<N, 1024, lds, (hipStream_t)stream>>>(
       (const half_t*)h, nullptr, nullptr, nullptr, nullptr, 0, nullptr, 0.f, (const half_t*)router, E, H, nullptr, nullptr,
       (half_t*)logits, nullptr, 0, front);
   return sy_check_launch("router_route_sort");
+}
+
+// The router GEMM and route for a few rows, one workgroup per row and no sort: what
+// sy_router_route does for a decode step (front.hip hands such calls over).
+int sy_router_route_rows(const void* h, const void* router, int N, int H, int E, int k, int norm, void* logits, int32_t* idx,
+                         void* w, void* stream) {
+  ROW_LIMITS("router_route");
+  SY_REQUIRE(E >= 1 && E <= 128 && k >= 1 && k <= front_core::TAIL_MAX_K && k <= E,
+             "router_route: at most 128 experts and top-8 (got E = %d, k = %d)", E, k);
+  if (N == 0) return SY_OK;
+  SY_REQUIRE(h && router && logits && idx && w, "router_route: null pointer");
+  front_core::Outputs front{idx, (half_t*)w, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, k, norm, 0};
+  const size_t lds = (size_t)H * sizeof(half_t) + sizeof(half_t) * ((size_t)(E + 7) / 8 * 8);
+  row_kernel<false, true, FRONT_ROUTE><<<N, 1024, lds, (hipStream_t)stream>>>(
+      (const half_t*)h, nullptr, nullptr, nullptr, nullptr, 0, nullptr, 0.f, (const half_t*)router, E, H, nullptr, nullptr,
+      (half_t*)logits, nullptr, 0, front);
+  return sy_check_launch("router_route");
 }
 
 extern "C" SY_API int sy_add_rmsnorm_route_sort(const void* x, const void* delta, const void* weight, float eps,
@@ -775,7 +797,7 @@ extern "C" SY_API int sy_add_rmsnorm_route_sort(const void* x, const void* delta
   const int rc = front_outputs("add_rmsnorm_route_sort", N, E, k, norm, idx, w, counts, offsets, token, wsorted, pos_of, &front);
   if (rc) return rc;
   const size_t lds = (size_t)H * sizeof(half_t) + front_core::tail_lds_bytes(N, E, k);
-  row_kernel<false, true, true><<<N, 1024, lds, (hipStream_t)stream>>>(
+  row_kernel<false, true, FRONT_SORT><<<N, 1024, lds, (hipStream_t)stream>>>(
       (const half_t*)x, (const half_t*)delta, nullptr, nullptr, nullptr, 0, (const half_t*)weight, eps,
       (const half_t*)router, E, H, (half_t*)x_out, (half_t*)h_out, (half_t*)logits, nullptr, 0, front);
   return sy_check_launch("add_rmsnorm_route_sort");

@@ -424,5 +424,7 @@ int sy_router_route_counting(const void* h, const void* router, int N, int H, in
 extern "C" SY_API int sy_router_route(const void* h, const void* router, int N, int H, int E, int k, int norm, void* logits,
                                       int32_t* idx, void* w, void* stream) {
   if (N == 0) return SY_OK;
+  // a decode step: one workgroup per row (the kernels above take 16 rows to a workgroup)
+  if (N <= 64) return sy_router_route_rows(h, router, N, H, E, k, norm, logits, idx, w, stream);
   return sy_router_route_counting(h, router, N, H, E, k, norm, logits, idx, w, nullptr, stream);
 }

@@ -45,6 +45,22 @@ __host__ __device__ constexpr size_t tail_lds_bytes(int N, int E, int k) {
          sizeof(half_t) * (size_t)N * k;
 }
 
+// The route alone, for a caller whose next launch sorts for itself (the weight stream of a decode
+// step of at most 64 choices does): the workgroup's first wavefront routes token t from the
+// logits at `lds`; nothing is counted and nobody sorts. Only idx and w of `o` are used.
+template <int PER_LANE>
+__device__ __forceinline__ void route_own(int t, int E, const Outputs& o, const unsigned char* lds) {
+  if ((threadIdx.x >> 6) != 0) return;
+  const int lane = threadIdx.x & 63;
+  int my_e;
+  float my_w;
+  route_core::route_token<half_t, PER_LANE>(reinterpret_cast<const half_t*>(lds), E, o.k, o.norm, my_e, my_w);
+  if (lane < o.k) {
+    o.idx[t * o.k + lane] = my_e;
+    o.w[t * o.k + lane] = (half_t)my_w;
+  }
+}
+
 // Called by every thread of a workgroup of SORT_THREADS threads whose token is t of N, after a
 // barrier behind which `lg` (the first E halves of `lds`) holds the token's logits.
 template <int PER_LANE>

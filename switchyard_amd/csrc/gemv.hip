@@ -29,7 +29,7 @@
 //
 // Replaces grouped_gemv_kernel / grouped_gemv of the reference
 // (switchyard/csrc/moe_kernels.cu:301-415); epilogue rounding points as :373-378.
-#include "common.h"
+#include "sort_core.h"
 
 namespace {
 
@@ -199,23 +199,70 @@ __device__ __forceinline__ void run_pass(const Pass& p) {
   }
 }
 
-template <bool SWIGLU, bool SCALE, bool EXACT, int CH>
+// What a launch that sorts for itself reads and leaves behind: the routing of at most 64 choices
+// (a decode step of 8 tokens) in, the five results of sort_by_expert out.
+struct SortHere {
+  const int* idx;        // [N, k]
+  const half_t* w;       // [N, k]
+  int M, k, nbits;
+  int* counts;           // [E]
+  int* offsets;          // [E + 1]
+  int* token;            // [M]
+  half_t* wsorted;       // [M]
+  int* pos_of;           // [M]
+};
+constexpr int SORT_HERE_MAX = WAVE;   // choices that one wavefront sorts with one per lane
+__host__ __device__ constexpr size_t sort_here_ints(int E) {
+  return (size_t)E + (E + 1) + 2 * SORT_HERE_MAX + SORT_HERE_MAX / 2 + (2 * E + 1);
+}
+
+// With SORT the launch has no sorted rows to start from, only the routing: every workgroup
+// sorts the (at most 64) choices itself, one wavefront with a choice per lane, into LDS, and
+// the first workgroup also writes the results out for the launches that follow. In front of a
+// weight stream of tens of microseconds that costs each workgroup a few hundred cycles where
+// its scan of `offsets` stood, and the launch before it need not gather every token's choices
+// in one place.
+template <bool SWIGLU, bool SCALE, bool EXACT, int CH, bool SORT = false>
 __global__ void __launch_bounds__(GEMV_THREADS)
 gemv_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const half_t* __restrict__ B,
             const int* __restrict__ offsets, int E, int Nout, int K, const half_t* __restrict__ scale,
-            half_t* __restrict__ C, int row_cap) {
+            half_t* __restrict__ C, int row_cap, SortHere sort = SortHere{}) {
   extern __shared__ __attribute__((aligned(16))) half_t xs[];  // [row_cap][K + ROW_PAD], then the used experts
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int RS = K + ROW_PAD;
   int* used = reinterpret_cast<int*>(xs + (size_t)row_cap * RS);  // [E] ids of experts with rows, [E] = how many
   const half8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  // SORT: the sort's results in LDS, behind the list of used experts
+  int* s_counts = used + E + 1;
+  int* s_offsets = s_counts + E;
+  int* s_token = s_offsets + E + 1;
+  int* s_pos = s_token + SORT_HERE_MAX;
+  uint16_t* s_wsorted = reinterpret_cast<uint16_t*>(s_pos + SORT_HERE_MAX);
+  if (SORT) {
+    if (wave == 0)
+      sort_core::sort_one_wave<uint16_t>(sort.idx, reinterpret_cast<const uint16_t*>(sort.w), sort.M, sort.k, E, sort.nbits,
+                                         s_counts, s_offsets, s_token, s_wsorted, s_pos,
+                                         reinterpret_cast<int*>(s_wsorted + SORT_HERE_MAX));
+    __syncthreads();
+    if (blockIdx.x == 0) {
+      for (int i = threadIdx.x; i <= E; i += GEMV_THREADS) {
+        sort.offsets[i] = s_offsets[i];
+        if (i < E) sort.counts[i] = s_counts[i];
+      }
+      for (int i = threadIdx.x; i < sort.M; i += GEMV_THREADS) {
+        sort.token[i] = s_token[i];
+        sort.pos_of[i] = s_pos[i];
+        reinterpret_cast<uint16_t*>(sort.wsorted)[i] = s_wsorted[i];
+      }
+    }
+  }
 
   // ---- the experts that received rows, in order (one wavefront, 64 experts per step)
   if (wave == 0) {
     int n = 0;
     for (int e0 = 0; e0 < E; e0 += WAVE) {
       const int e = e0 + lane;
-      const bool has = e < E && offsets[e + 1] > offsets[e];
+      const bool has = e < E && (SORT ? s_offsets[e + 1] > s_offsets[e] : offsets[e + 1] > offsets[e]);
       const uint64_t m = __ballot(has);
       if (has) used[n + __popcll(m & lanemask_lt())] = e;
       n += __popcll(m);
@@ -246,7 +293,7 @@ gemv_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const 
     const int u = at / units_per_expert, first = at - u * units_per_expert;
     const int count = min(hi - at, units_per_expert - first);
     const int e = used[u];
-    const int start = offsets[e], end = offsets[e + 1];
+    const int start = SORT ? s_offsets[e] : offsets[e], end = SORT ? s_offsets[e + 1] : offsets[e + 1];
     p.rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(B + (size_t)e * Nfull * K), 0,
                                                (int)((size_t)Nfull * K * 2), 0x00020000);
     // wavefront w takes a contiguous quarter of the units
@@ -259,7 +306,7 @@ gemv_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const 
       // ---- stage the pass's rows: wavefront w copies rows w, w+4, ...; missing rows of the last quad are zero
       if (staged) __syncthreads();
       for (int r = wave; r < nq * QUAD; r += GEMV_WAVES) {
-        const half_t* src = r < nr ? A + (size_t)(a_rows ? a_rows[r0 + r] : r0 + r) * K : nullptr;
+        const half_t* src = r < nr ? A + (size_t)(SORT ? s_token[r0 + r] : a_rows ? a_rows[r0 + r] : r0 + r) * K : nullptr;
         for (int kk = lane * 8; kk < K; kk += WAVE * 8)
           *reinterpret_cast<half8_t*>(xs + r * RS + kk) = src ? *reinterpret_cast<const half8_t*>(src + kk) : zero8;
       }
@@ -279,13 +326,15 @@ gemv_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const 
 }
 
 int launch_gemv(const void* A, const int32_t* a_rows, const void* B, const int32_t* offsets, int E, int rows,
-                int max_rows_hint, int Nout, int K, int swiglu, const void* scale, void* C, hipStream_t stream) {
+                int max_rows_hint, int Nout, int K, int swiglu, const void* scale, void* C, hipStream_t stream,
+                const SortHere* sort = nullptr) {
   // rows staged per pass: no expert has more rows than there are rows in all; a caller that
   // knows a tighter bound (the number of tokens) saves LDS and gains occupancy
   const int bound = max_rows_hint > 0 && max_rows_hint < rows ? max_rows_hint : rows;
   int row_cap = (bound + QUAD - 1) / QUAD * QUAD;
   row_cap = row_cap > MAX_QUADS * QUAD ? MAX_QUADS * QUAD : row_cap;
-  const size_t lds = (size_t)row_cap * (K + ROW_PAD) * sizeof(half_t) + (size_t)(E + 1) * sizeof(int);
+  const size_t lds = (size_t)row_cap * (K + ROW_PAD) * sizeof(half_t) + (size_t)(E + 1) * sizeof(int) +
+                     (sort ? sort_here_ints(E) * sizeof(int) : 0);
   // Loads in flight per wavefront: a chunk of 4 KB, or of 8 KB where a unit is long enough to be
   // cut into such chunks (gate and up rows of 2048 at 8 tokens: 56.6 us against 57.5; for rows of
   // 1024 the longer chunk is one per unit and loses: 34.8 us against 30.6).
@@ -307,19 +356,43 @@ int launch_gemv(const void* A, const int32_t* a_rows, const void* B, const int32
   const half_t* b = (const half_t*)B;
   const half_t* s = (const half_t*)scale;
   half_t* c = (half_t*)C;
-  void (*kern)(const half_t*, const int*, const half_t*, const int*, int, int, int, const half_t*, half_t*, int);
-  if (swiglu && long_chunks && exact) kern = gemv_kernel<true, false, true, CH_LONG>;
+  void (*kern)(const half_t*, const int*, const half_t*, const int*, int, int, int, const half_t*, half_t*, int, SortHere);
+  if (sort && long_chunks && exact) kern = gemv_kernel<true, false, true, CH_LONG, true>;
+  else if (sort) kern = exact ? gemv_kernel<true, false, true, CH_SHORT, true> : gemv_kernel<true, false, false, CH_SHORT, true>;
+  else if (swiglu && long_chunks && exact) kern = gemv_kernel<true, false, true, CH_LONG>;
   else if (swiglu) kern = exact ? gemv_kernel<true, false, true, CH_SHORT> : gemv_kernel<true, false, false, CH_SHORT>;
   else if (s) kern = exact ? gemv_kernel<false, true, true, CH_SHORT> : gemv_kernel<false, true, false, CH_SHORT>;
   else kern = exact ? gemv_kernel<false, false, true, CH_SHORT> : gemv_kernel<false, false, false, CH_SHORT>;
   hipError_t attr = hipSuccess;
   if (lds > 48 * 1024) attr = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (attr != hipSuccess) return sy_fail(SY_ERR_LAUNCH, "grouped_gemv: cannot reserve %zu bytes of LDS", lds);
-  kern<<<(unsigned)grid, GEMV_THREADS, lds, stream>>>(a, a_rows, b, offsets, E, Nout, K, swiglu ? nullptr : s, c, row_cap);
+  kern<<<(unsigned)grid, GEMV_THREADS, lds, stream>>>(a, a_rows, b, offsets, E, Nout, K, swiglu ? nullptr : s, c, row_cap,
+                                                      sort ? *sort : SortHere{});
   return sy_check_launch("grouped_gemv");
 }
 
 }  // namespace
+
+// The gate/up projection (SwiGLU) of a decode step straight from the routing: sort_by_expert of
+// at most 64 choices happens inside the launch, whose first workgroup also writes the sort's
+// five results for the launches behind it. Same `act` as sy_sort_by_expert followed by
+// sy_grouped_gemv, bit for bit.
+int sy_grouped_gemv_sorting(const void* h, const int32_t* idx, const void* w, int N, int k, const void* gate_up, int E, int I,
+                            int H, int32_t* counts, int32_t* offsets, int32_t* token, void* wsorted, int32_t* pos_of,
+                            void* act, void* stream) {
+  SY_REQUIRE(sy_gemv_sorts(N, k, E, H), "grouped_gemv_sorting: N = %d, k = %d, E = %d, H = %d", N, k, E, H);
+  SY_REQUIRE((long)2 * I * H * 2 < (1l << 31) && I >= 1, "grouped_gemv_sorting: an expert's matrix must stay under 2 GiB");
+  SY_REQUIRE(h && idx && w && gate_up && counts && offsets && token && wsorted && pos_of && act, "grouped_gemv_sorting: null pointer");
+  int nbits = 0;
+  while ((1 << nbits) < E) ++nbits;
+  const SortHere sort{idx, (const half_t*)w, N * k, k, nbits, counts, offsets, token, (half_t*)wsorted, pos_of};
+  return launch_gemv(h, nullptr, gate_up, nullptr, E, N * k, N, I, H, 1, nullptr, act, (hipStream_t)stream, &sort);
+}
+
+// Whether sy_grouped_gemv_sorting takes this shape: one choice per lane of a wavefront.
+bool sy_gemv_sorts(int N, int k, int E, int H) {
+  return N >= 1 && k >= 1 && (long)N * k <= SORT_HERE_MAX && E >= 1 && E <= 128 && k <= E && H >= 8 && H % 8 == 0 && H <= 4096;
+}
 
 extern "C" SY_API int sy_grouped_gemv(const void* A, const int32_t* a_rows, const void* B, const int32_t* offsets,
                                       int E, int rows, int max_rows_hint, int Nout, int K, int swiglu,

@@ -123,9 +123,15 @@ def experts(h, idx, w, gate_up, down, mode="auto"):
     E = ext()
     N = h.shape[0]
     idx = idx.contiguous()
-    counts, offsets, token, wsorted, pos_of = E.sort_by_expert(idx, w.contiguous(), gate_up.shape[0])
     if mode == "auto":
         mode = _auto(N, idx.numel(), gate_up.shape[0])
+    if mode not in ("gemv", "gemm", "cublas"):
+        raise ValueError(f"unknown mode {mode!r}")
+    if (N > 0 and h.dtype == torch.float16 and w.dtype == torch.float16 and gate_up.shape[0] <= 512
+            and idx.shape[1] <= 64 and N * h.shape[1] * 2 < 2 ** 31):
+        # one call of the library: the host pays per call what the GPU needs for a small kernel
+        return E.experts_routed(h.contiguous(), idx, w.contiguous(), gate_up, down, mfma_tiles=mode != "gemv")
+    counts, offsets, token, wsorted, pos_of = E.sort_by_expert(idx, w.contiguous(), gate_up.shape[0])
     y = ffn(h, token, offsets, counts, wsorted, gate_up, down, idx.numel(), mode)
     return E.combine(y, pos_of, idx, N)
 

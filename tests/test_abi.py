@@ -32,7 +32,7 @@ def test_header_declares_the_expected_entry_points():
                                                            "sy_router_route_sort"]
     assert sorted(os.listdir(os.path.join(ROOT, "include"))) == ["switchyard_decode.h", "switchyard_moe.h"]
     assert sorted(declared_symbols(HEADER)) == sorted(["sy_version", "sy_last_error", "sy_route", "sy_sort_workspace_bytes",
-                                                  "sy_sort_by_expert", "sy_sort_by_expert_static", "sy_route_sort", "sy_router_route", "sy_experts_sorted",
+                                                  "sy_sort_by_expert", "sy_sort_by_expert_static", "sy_route_sort", "sy_router_route", "sy_experts_sorted", "sy_experts_routed",
                                                   "sy_grouped_gemv", "sy_grouped_gemm",
                                                   "sy_combine", "sy_moe_experts"])
 

@@ -640,3 +640,53 @@ def test_moe_experts_entry_point_with_a_router_at_decode_sizes(K, N, tiles):
     assert torch.equal(idx, ridx) and torch.equal(w, rw)
     for a, b in zip((counts, offsets, token, wsorted, pos_of), ext.sort_by_expert(ridx, rw, E)):
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("N,E,k,H,I", [(1, 64, 8, 2048, 1024), (8, 64, 8, 2048, 1024), (5, 16, 4, 128, 64), (3, 128, 8, 520, 72),
+                                       (64, 64, 1, 256, 128), (7, 60, 3, 1024, 256),
+                                       (9, 64, 8, 512, 128), (300, 64, 8, 256, 128)])   # these two sort in a launch of their own
+@pytest.mark.parametrize("tiles", [False, True])
+def test_experts_from_the_routing_in_one_call(K, N, E, k, H, I, tiles):
+    """sy_experts_routed is experts() of the reference in one call. Up to 64 choices on the
+    weight-stream kernels the gate/up launch sorts for itself: the sort's five results and
+    `out` are bit for bit those of sort_by_expert, the two projections and combine."""
+    if tiles and (H % 32 or I % 32):
+        pytest.skip("the MFMA tiles need K % 32 == 0, as the reference's do")
+    h, router, gu, dn = (t.to(DEV) for t in cases.layer(N, E=E, k=k, H=H, I=I, seed=6, wstd=0.05))
+    ext = K.ext()
+    idx, w = ext.route(F.linear(h, router).contiguous(), k, True)
+    want_sort = ext.sort_by_expert(idx, w, E)
+    counts, offsets, token, wsorted, pos_of = want_sort
+    want = ext.combine(K.ffn(h, token, offsets, counts, wsorted, gu, dn, N * k, "gemm" if tiles else "gemv"), pos_of, idx, N)
+    assert torch.equal(K.experts(h, idx, w, gu, dn, "gemm" if tiles else "gemv"), want)   # experts() takes the one call
+    M = N * k
+    i32 = dict(dtype=torch.int32, device=DEV)
+    f16 = dict(dtype=torch.float16, device=DEV)
+    counts, offsets = torch.empty(E, **i32), torch.empty(E + 1, **i32)
+    token, wsorted, pos_of = torch.empty(M, **i32), torch.empty(M, **f16), torch.empty(M, **i32)
+    act, y, out = torch.empty(M, I, **f16), torch.empty(M, H, **f16), torch.empty(N, H, **f16)
+    need = ext.lib.sy_sort_workspace_bytes(N, k, E)
+    ws = torch.empty(max(need, 1), dtype=torch.uint8, device=DEV)
+    for _ in range(2):
+        rc = ext.lib.sy_experts_routed(h.data_ptr(), N, E, k, gu.data_ptr(), dn.data_ptr(), H, I, int(tiles), idx.data_ptr(),
+                                       w.data_ptr(), counts.data_ptr(), offsets.data_ptr(), token.data_ptr(),
+                                       wsorted.data_ptr(), pos_of.data_ptr(), act.data_ptr(), y.data_ptr(), out.data_ptr(),
+                                       ws.data_ptr(), need, torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, ext.lib.sy_last_error()
+        assert torch.equal(out, want)
+        for a, b in zip((counts, offsets, token, wsorted, pos_of), want_sort):
+            assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("N,E,k,H", [(1, 64, 8, 2048), (8, 64, 8, 2048), (64, 64, 8, 2048), (5, 100, 5, 520), (64, 128, 8, 8192)])
+def test_router_route_at_decode_sizes(K, N, E, k, H):
+    """Up to 64 tokens sy_router_route is a workgroup per token: the logits of router_logits and
+    the ids and weights of route on them, bit for bit."""
+    g = torch.Generator().manual_seed(N + E)
+    h = torch.randn(N, H, generator=g).half().to(DEV)
+    router = (torch.randn(E, H, generator=g) * H ** -0.5).half().to(DEV)
+    ext = K.ext()
+    idx, w, logits = ext.router_route(h, router, k, True)
+    assert torch.equal(logits, ext.router_logits(h, router))
+    ridx, rw = ext.route(logits, k, True)
+    assert torch.equal(idx, ridx) and torch.equal(w, rw)
