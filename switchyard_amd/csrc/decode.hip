@@ -115,7 +115,7 @@ row_kernel(const half_t* x, const half_t* __restrict__ delta, const half_t* __re
       if (COMBINE) {
         float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         for (int j = 0; j < k; ++j) {
-          const half8_t e = *reinterpret_cast<const half8_t*>(y + (size_t)rows[j] * H + c * 8);
+          const half8_t e = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(y + (size_t)rows[j] * H + c * 8));   // read once
           const float wt = wts[j];
           // the rounding of the down projection's scaled epilogue (times 1 it changes nothing)
 #pragma unroll
@@ -437,8 +437,8 @@ decode_attention_kernel(const half_t* __restrict__ q, const half_t* kcache, cons
       kb.kk[u] = zero8;
       kb.vv[u] = zero8;
       if (kb.ok[u]) {
-        kb.kk[u] = *reinterpret_cast<const half8_t*>(kcache + base + (size_t)key * D);
-        kb.vv[u] = *reinterpret_cast<const half8_t*>(vcache + base + (size_t)key * D);
+        kb.kk[u] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(kcache + base + (size_t)key * D));   // the cache is
+        kb.vv[u] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(vcache + base + (size_t)key * D));   // read once a step
         kb.ok[u] = rl[key] != 0;
       }
     }

@@ -13,8 +13,6 @@ Differences that follow from the hardware, none visible in the results:
     "cublas" is still accepted and runs the MFMA kernel.
 """
 
-import math
-
 import torch
 import torch.nn.functional as F
 
@@ -68,29 +66,24 @@ def pick(max_rows):
     return "gemm"
 
 
-# Above this many tokens "auto" never takes the weight-stream kernel: it handles 16 rows of an
-# expert per pass, a token picks an expert at most once, so up to 16 tokens one pass is certain
-# whatever the routing. Beyond that a popular expert takes a second pass and its many rows make
-# the stream compute-bound. Measured (us per experts() call, stream of calls; Zipf bias with
-# every token on the most popular expert): 17 tokens balanced 128 (gemv) / 135 (gemm), Zipf
-# 96 / 75; 24 tokens balanced 139 / 143, Zipf 125 / 87; 32 tokens balanced 147 / 146, Zipf
-# 160 / 111. Without a device read the routing is unknown, and what the MFMA tiles lose under
-# balanced routing (0 to 6 %) is small against what the stream loses under skew (20 to 30 %).
-GEMV_MAX_TOKENS = 16
+# Above this many tokens "auto" never takes the weight-stream kernel. Up to GEMV_MAX_ROWS tokens
+# no expert can have more rows than that, whatever the routing, and the weight stream wins (8
+# tokens: 88.7 us for the two projections against 95.8 on the MFMA tiles, whose one workgroup
+# per tile leaves a third of the CUs' slots empty with 41 used experts). Above, the MFMA tiles
+# with their weights loaded non-temporal stream faster than the weight-stream kernel does (12
+# tokens 102.4 against 107.2 us, 16 tokens 106.3 against 113.0, 32 tokens 119.8 against 133.4:
+# 6.5 to 6.6 TB/s against 6.0 to 6.2), and they do not slow down when a popular expert collects
+# many rows (Zipf routing cost the weight stream 20 to 30 % at 17 to 32 tokens).
+GEMV_MAX_TOKENS = 8
 
 
 def _auto(n_tokens, n_choices, n_experts):
-    """Mode for "auto" without a device read. No expert can have more rows than there are
-    tokens, so up to GEMV_MAX_ROWS tokens the answer is certain; up to GEMV_MAX_TOKENS the
-    busiest expert is estimated from the mean rows per expert (under near-uniform routing it
-    sits about two square roots of the mean above it); beyond, the MFMA tiles. Both kernels
-    are correct for any routing."""
-    if n_tokens <= GEMV_MAX_ROWS:
+    """Mode for "auto" without a device read: the weight stream while no expert can have more
+    than GEMV_MAX_ROWS rows (at most that many tokens), else the MFMA tiles. Both kernels are
+    correct for any routing."""
+    if n_tokens <= min(GEMV_MAX_ROWS, GEMV_MAX_TOKENS):
         return "gemv"
-    if n_tokens > GEMV_MAX_TOKENS:
-        return "gemm"
-    mean = n_choices / n_experts
-    return pick(math.ceil(mean + 2.0 * math.sqrt(mean)))
+    return "gemm"
 
 
 def ffn(x, a_rows, offsets, counts, wsorted, gate_up, down, rows, mode, host_counts=None):
