@@ -10,8 +10,9 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB = None
 
 
-def build():
-    subprocess.run(["make", "-s", "-C", _HERE, "liboracle_moe.so"], check=True)
+def build(force=False):
+    """Compile the C restatement; force=True compiles also where a built library is there."""
+    subprocess.run(["make", "-s"] + (["-B"] if force else []) + ["-C", _HERE, "liboracle_moe.so"], check=True)
 
 
 def lib():
