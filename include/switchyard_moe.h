@@ -11,8 +11,9 @@
  *   - "f16" is IEEE binary16; every matrix is row-major and contiguous;
  *   - the return value is 0 on success, otherwise an SY_ERR_* code, and sy_last_error()
  *     returns a message for the calling thread;
- *   - calls are re-entrant and the library keeps no state between calls (the one exception,
- *     sy_sort_by_expert_static, says so).
+ *   - calls are re-entrant and the library keeps no state between calls (the exceptions say so:
+ *     sy_sort_by_expert_static's workspace, and the launch counters of sy_router_route_sort and
+ *     sy_add_rmsnorm_route_sort in switchyard_decode.h).
  */
 #ifndef SWITCHYARD_MOE_H
 #define SWITCHYARD_MOE_H
