@@ -320,7 +320,7 @@ gemm_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const 
 // read), so the waits are written by hand.
 constexpr int BIG_BM = 256;
 constexpr int BIG_BK = 64;                                        // K per slice
-constexpr int BIG_STEPS = BIG_BK / 16;                            // MFMA K-steps per slice
+constexpr int BIG_STEPS = BIG_BK / 32;                            // MFMA K-steps per slice
 constexpr int BIG_ROW_BYTES = BIG_BK * 2;                         // 128
 constexpr int BIG_A_BYTES = BIG_BM * BIG_ROW_BYTES;               // 32 KB: a slice of the rows
 constexpr int BIG_B_BYTES = BW * BIG_ROW_BYTES;                   // 32 KB: a slice of the weight rows
@@ -386,28 +386,33 @@ __device__ __forceinline__ void scalar_load_4x8(const int* p0, const int* p1, co
 }
 
 typedef int int16v_t __attribute__((ext_vector_type(16)));
-// scale[first + l] for l = 0..31 (first is the same in the whole wavefront): 17 dwords from the
-// dword at or below scale + first through the scalar cache, waited for here; a lane picks its
-// half. The run is moved up where it would pass the end of the M scales (M >= 34); lanes whose
-// row is past the end get whatever is there.
-__device__ __forceinline__ half_t scale_of_row(const half_t* scale, int M, int first, int l) {
+// scale[first + l] and scale[first + 16 + l] for l = 0..15 (first is the same in the whole
+// wavefront): 17 dwords from the dword at or below scale + first through the scalar cache, waited
+// for here; a lane picks its two halves. The run is moved up where it would pass the end of the M
+// scales (M >= 34); lanes whose row is past the end get whatever is there.
+__device__ __forceinline__ void scales_of_rows(const half_t* scale, int M, int first, int l, half_t& lo16, half_t& hi16) {
   const uint64_t want = (uint64_t)(scale + first), end = ((uint64_t)(scale + M) + 3) & ~(uint64_t)3;
   uint64_t from = want & ~(uint64_t)3;
   from = from < end - 68 ? from : end - 68;
   const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)from), hi = __builtin_amdgcn_readfirstlane((unsigned)(from >> 32));
   from = ((uint64_t)hi << 32) | lo;
   int16v_t words;
-  int word;
+  int last;
   asm volatile(
       "s_load_dwordx16 %0, %2, 0x0\n\t"
       "s_load_dword %1, %2, 0x40\n\t"
       "s_waitcnt lgkmcnt(0)"
-      : "=&s"(words), "=&s"(word)
+      : "=&s"(words), "=&s"(last)
       : "s"((const unsigned*)from));
-  const int h = (int)((want - from) >> 1) + l;
+  auto pick = [&](int h) {
+    int word = last;
 #pragma unroll
-  for (int d = 0; d < 16; ++d) word = (h >> 1) == d ? words[d] : word;
-  return __builtin_bit_cast(half_t, (unsigned short)((h & 1) ? (unsigned)word >> 16 : (unsigned)word));
+    for (int d = 0; d < 16; ++d) word = (h >> 1) == d ? words[d] : word;
+    return __builtin_bit_cast(half_t, (unsigned short)((h & 1) ? (unsigned)word >> 16 : (unsigned)word));
+  };
+  const int h = (int)((want - from) >> 1) + l;
+  lo16 = pick(h);
+  hi16 = pick(h + 16);
 }
 
 template <int EPL>
@@ -432,9 +437,8 @@ gemm_stream_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows,
                    const int* __restrict__ offsets, int E, int M, int Nout, int K, const half_t* __restrict__ scale,
                    half_t* __restrict__ C, int ncol_tiles) {
   constexpr int BM = BIG_BM, WN = 4;
-  constexpr bool TURN = !SWIGLU;   // outputs turned round in LDS for whole-row stores (see the epilogue)
   constexpr int WAVES = 2 * WN, THREADS = WAVES * WAVE;
-  constexpr int NB = BW / (32 * WN);
+  constexpr int WB = BW / (16 * WN);   // blocks of 16 weight rows per wavefront
   constexpr int LOADS = BIG_A_BYTES / (THREADS * 16);
   __shared__ __attribute__((aligned(1024))) char lds[BIG_A_STAGES * BIG_A_BYTES + BIG_B_STAGES * BIG_B_BYTES];
   const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
@@ -609,16 +613,21 @@ gemm_stream_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows,
   };
 
   const int wm = wave / WN, wn = wave % WN;
-  const int l32 = lane & 31;
-  int brow[NB];
+  // v_mfma_f32_16x16x32_f16: a lane gives 8 consecutive K of row (lane & 15), the four groups of
+  // 16 lanes cover the 32 K of a step, and ends with 4 consecutive weight rows (output columns),
+  // 4 * (lane >> 4) + 0..3, of row (lane & 15). A wavefront's 128 rows x 64 weight rows are 8 x 4
+  // such blocks. (On random operands this shape sustains 16 % more flops than 32x32x16 under the
+  // chip's power management: 2.0 against 1.72 Pflop/s in a loop of MFMAs alone.)
+  const int l16 = lane & 15, lg = lane >> 4;
+  int brow[WB];
 #pragma unroll
-  for (int j = 0; j < NB; ++j)
-    brow[j] = SWIGLU ? (j < NB / 2 ? 0 : COLS) + wn * (NB / 2 * 32) + (j % (NB / 2)) * 32 : wn * (NB * 32) + j * 32;
+  for (int j = 0; j < WB; ++j)
+    brow[j] = SWIGLU ? (j < WB / 2 ? 0 : COLS) + wn * (WB / 2 * 16) + (j % (WB / 2)) * 16 : wn * (WB * 16) + j * 16;
   int koff[BIG_STEPS];
 #pragma unroll
-  for (int s = 0; s < BIG_STEPS; ++s) koff[s] = (((2 * s + (lane >> 5)) ^ ((l32 >> 1) & 7)) * 16);
-  const char* as = lds + (wm * 32 + l32) * BIG_ROW_BYTES;
-  const char* bs = lds + BIG_A_STAGES * BIG_A_BYTES + l32 * BIG_ROW_BYTES;
+  for (int s = 0; s < BIG_STEPS; ++s) koff[s] = (((4 * s + lg) ^ (l16 >> 1)) * 16);
+  const char* as = lds + (wm * 32 + l16) * BIG_ROW_BYTES;
+  const char* bs = lds + BIG_A_STAGES * BIG_A_BYTES + l16 * BIG_ROW_BYTES;
 
   // ---- fill the pipe for the first tile: rows 0, weights 0 | rows 1, weights 1 (the first
   // iteration asks for weights 2)
@@ -633,68 +642,111 @@ gemm_stream_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows,
   __syncthreads();
   int a_stage = 0, b_stage = 0;  // where the current tile's slice 0 is
 
-  float16_t acc[4][NB];
+  float4_t acc[8][WB];   // [16-row unit ib: rows (2 (ib / 2) + wm) * 32 + (ib % 2) * 16 ..][16 weight rows jb]
   for (;;) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 8; ++i)
 #pragma unroll
-      for (int j = 0; j < NB; ++j)
+      for (int j = 0; j < WB; ++j)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+        for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
 
     // On entry slice 0 of the current tile has landed and every wavefront knows it.
+    //
+    // A slice is two K-steps of 2 * LIVE units; a unit is the 4 MFMAs of one 16-row block against
+    // the wavefront's 4 blocks of weight rows, and a quarter of a slice is LIVE units. The weight
+    // operands of a K-step live in registers for the whole step (two sets: the next step's are
+    // read during the second quarter of this one). The row operands go through a ring: the read
+    // for the unit one quarter ahead goes into the slot that a unit of this quarter has just left
+    // (LIVE >= 3; with fewer units the ring has two quarters, so that a read is not issued only
+    // one unit before its use). Reads never run more than a quarter ahead, because the barrier
+    // before the last quarter is what publishes the next slice and frees this one's buffers.
     auto k_loop = [&](auto live_blocks) {
       constexpr int LIVE = decltype(live_blocks)::value;
-      constexpr int READS = LIVE > 0 ? LIVE + NB : 0, MFMAS = NB * LIVE;
-      constexpr int PAIRS = READS < MFMAS ? READS : MFMAS;
-      half8_t xf[2][LIVE > 0 ? LIVE : 1], wf[2][NB];
-      auto read = [&](int sa, int sb, int s, int r) {
-        if (r < NB) wf[s & 1][r] = *reinterpret_cast<const half8_t*>(bs + sb + brow[r] * BIG_ROW_BYTES + koff[s]);
-        else xf[s & 1][r - NB] = *reinterpret_cast<const half8_t*>(as + sa + (r - NB) * 64 * BIG_ROW_BYTES + koff[s]);
+      constexpr int QU = LIVE, NU = 2 * LIVE;          // units per quarter, per K-step
+      constexpr int R = LIVE >= 3 ? LIVE : 2 * LIVE;   // slots of the ring
+      half8_t xr[R > 0 ? R : 1], wf[2][WB];
+      auto read_x = [&](int sa, int g) {   // unit g of a slice (0 .. 4 LIVE - 1) into its slot
+        const int s = (g / (NU > 0 ? NU : 1)) & 1, ib = g % (NU > 0 ? NU : 1);
+        xr[g % (R > 0 ? R : 1)] =
+            *reinterpret_cast<const half8_t*>(as + sa + ((ib >> 1) * 64 + (ib & 1) * 16) * BIG_ROW_BYTES + koff[s]);
       };
-      auto mfma = [&](int s, int m) {
-        const int i = m / NB, j = m % NB;
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[s & 1][j], xf[s & 1][i], acc[i][j], 0, 0, 0);
+      auto read_w = [&](int sb, int s, int j) {
+        wf[s][j] = *reinterpret_cast<const half8_t*>(bs + sb + brow[j] * BIG_ROW_BYTES + koff[s]);
       };
+      auto mfma = [&](int g, int j) {
+        const int s = (g / (NU > 0 ? NU : 1)) & 1, ib = g % (NU > 0 ? NU : 1);
+        acc[ib][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf[s][j], xr[g % (R > 0 ? R : 1)], acc[ib][j], 0, 0, 0);
+      };
+      if constexpr (LIVE > 0) {
 #pragma unroll
-      for (int r = 0; r < READS; ++r) read(a_stage * BIG_A_BYTES, b_stage * BIG_B_BYTES, 0, r);
+        for (int j = 0; j < WB; ++j) read_w(b_stage * BIG_B_BYTES, 0, j);
+#pragma unroll
+        for (int u = 0; u < QU; ++u) read_x(a_stage * BIG_A_BYTES, u);
+      }
       for (int kt = 0; kt < nk; ++kt) {
         const int a_next = a_stage ^ 1, b_next = b_stage == BIG_B_STAGES - 1 ? 0 : b_stage + 1;
         const int b_free = b_stage == 0 ? BIG_B_STAGES - 1 : b_stage - 1;   // the buffer slice kt - 1 has left
         const int sa = a_stage * BIG_A_BYTES, sb = b_stage * BIG_B_BYTES;
         // A compute unit takes a load of this kind every 25 to 40 cycles, and a wavefront whose
         // load is not taken issues no MFMA either: the eight loads of an iteration are spread over
-        // it, the weights (slice kt + 2) one or two after each of the first three steps, the rows
-        // after the barrier, instead of all 64 of the workgroup at once.
+        // it, the weights (slice kt + 2) one or two after each of the first three quarters, the
+        // rows after the barrier, instead of all 64 of the workgroup at once.
 #pragma unroll
-        for (int s = 0; s < BIG_STEPS - 1; ++s) {
+        for (int q = 0; q < 3; ++q) {
+          if constexpr (LIVE > 0) {
 #pragma unroll
-          for (int r = 0; r < READS; ++r) read(sa, sb, s + 1, r);
+            for (int u = 0; u < QU; ++u) {
+              if (q == 1) {   // the second K-step's weight operands
 #pragma unroll
-          for (int m = 0; m < MFMAS; ++m) mfma(s, m);
+                for (int j = 0; j < WB; ++j)
+                  if (j * QU / WB == u) {
+                    read_w(sb, 1, j);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                  }
+              }
 #pragma unroll
-          for (int n = 0; n < PAIRS; ++n) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+              for (int j = 0; j < WB; ++j) mfma(q * QU + u, j);
+              read_x(sa, (q + 1) * QU + u);
+              if (R == LIVE) {
+                __builtin_amdgcn_sched_group_barrier(0x008, WB, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+              } else {
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, WB, 0);
+              }
+            }
           }
-          if (READS > PAIRS) __builtin_amdgcn_sched_group_barrier(0x100, READS - PAIRS, 0);
-          if (MFMAS > PAIRS) __builtin_amdgcn_sched_group_barrier(0x008, MFMAS - PAIRS, 0);
           __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-          for (int q = 0; q < LOADS; ++q)
-            if (q * (BIG_STEPS - 1) / LOADS == s) issue_weights(kt + 2, b_free, q);
+          for (int l = 0; l < LOADS; ++l)
+            if (l * 3 / LOADS == q) issue_weights(kt + 2, b_free, l);
           __builtin_amdgcn_sched_barrier(0);
         }
         asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(LOADS) : "memory");
         __syncthreads();
+        // the last quarter, in LOADS parts with a load of rows (slice kt + 2) behind each; it reads
+        // the first operands of the next slice
 #pragma unroll
         for (int part = 0; part < LOADS; ++part) {
+          if constexpr (LIVE > 0) {
 #pragma unroll
-          for (int r = 0; r < READS; ++r)
-            if (r * LOADS / (READS > 0 ? READS : 1) == part) read(a_next * BIG_A_BYTES, b_next * BIG_B_BYTES, 0, r);
+            for (int j = 0; j < WB; ++j)
+              if (j * LOADS / WB / 2 == part) read_w(b_next * BIG_B_BYTES, 0, j);
+            if (R != LIVE) {
 #pragma unroll
-          for (int m = 0; m < MFMAS; ++m)
-            if (m * LOADS / (MFMAS > 0 ? MFMAS : 1) == part) mfma(BIG_STEPS - 1, m);
+              for (int u = 0; u < QU; ++u)
+                if (4 * u / QU == part) read_x(a_next * BIG_A_BYTES, u);
+            }
+#pragma unroll
+            for (int m = 0; m < QU * WB; ++m)
+              if (m * LOADS / (QU * WB) == part) mfma(3 * QU + m / WB, m % WB);
+            if (R == LIVE) {
+#pragma unroll
+              for (int u = 0; u < QU; ++u)
+                if ((WB * u + WB - 1) * LOADS / (QU * WB) == part) read_x(a_next * BIG_A_BYTES, u);
+            }
+          }
           __builtin_amdgcn_sched_barrier(0);
           issue_rows(kt + 2, a_stage, part);
           __builtin_amdgcn_sched_barrier(0);
@@ -715,21 +767,24 @@ gemm_stream_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows,
       case 1: k_loop(std::integral_constant<int, 1>{}); break;
       default: k_loop(std::integral_constant<int, 0>{}); break;
     }
-    if constexpr (TURN) {
-      // ---- epilogue with whole-row stores (the projections without SwiGLU: a wavefront's share of
-      // a row is 64 columns, one 128-byte line). An accumulator block has a row per lane and 8
-      // bytes of it per store, so a store instruction would write 32 pieces of 16 bytes, and half
-      // of the launch's L2 requests would be such pieces. The weight buffer that the tile's last
-      // slice has just left stays free until the epilogue is done (its load, the next tile's
-      // third slice of weights, is issued below instead of in the last iteration), and each
-      // wavefront turns its outputs round in the four 1 KB pieces of it that its own loads fill:
-      // written 8 bytes per lane, the 8-byte slot XOR-ed with half the row number so that the 32
-      // rows of a block fall into different banks, read back 16 bytes per lane, 8 lanes to a row,
-      // and stored as 8 full lines per instruction.
-      const int last_stage = b_stage == 0 ? BIG_B_STAGES - 1 : b_stage - 1;   // b_stage already points at the next tile's slice 0
-      char* turn = lds + BIG_A_STAGES * BIG_A_BYTES + last_stage * BIG_B_BYTES + wave * 1024;   // piece c at + c * 8 KB
-      const int hsel = lane >> 5;
-      // the tile's columns all exist and rows of C are 16-byte aligned: no column is checked
+    // ---- epilogue. A lane holds 4 consecutive columns (8 bytes as f16) of its row in each of the
+    // wavefront's blocks of 16 columns, and the lane 16 further on the next 4. Two neighbouring
+    // blocks swap halves between those lanes (v_permlane16_swap), after which every lane holds 16
+    // consecutive bytes and a store instruction writes 64 consecutive bytes of each of 16 rows.
+    // No LDS is involved, so the stream's loads run on into the next tile meanwhile.
+    {
+      const int cofs = (lg & 1) * 16 + (lg >> 1) * 8;   // where a lane's 8 columns start after the swap
+      auto swap_halves = [&](half4_t a, half4_t b) -> half8_t {
+        typedef unsigned u2_t __attribute__((ext_vector_type(2)));
+        const u2_t ua = __builtin_bit_cast(u2_t, a), ub = __builtin_bit_cast(u2_t, b);
+        const auto lo = __builtin_amdgcn_permlane16_swap(ua[0], ub[0], false, false);
+        const auto hi = __builtin_amdgcn_permlane16_swap(ua[1], ub[1], false, false);
+        // lane group 0: a of groups 0 and 1 (columns 0..7 of the first block); group 1: b of groups
+        // 0 and 1 (columns 0..7 of the second block); groups 2 and 3 the same for columns 8..15
+        typedef unsigned u4_t __attribute__((ext_vector_type(4)));
+        const u4_t v = {lo[0], hi[0], lo[1], hi[1]};
+        return __builtin_bit_cast(half8_t, v);
+      };
       auto blocks = [&](auto whole_columns) {
         constexpr bool WHOLE = decltype(whole_columns)::value;
 #pragma unroll
@@ -738,80 +793,78 @@ gemm_stream_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows,
           if (rblock >= cur.row_end) continue;   // the same for the whole wavefront
           // the block's 32 scales come through the scalar cache: a vector load here would have to be
           // waited for, and with it every load of the stream that is in flight and every store so far
-          const half_t sc = SCALE ? scale_of_row(scale, M, rblock, l32) : (half_t)1.f;
-          const half4_t sc4 = {sc, sc, sc, sc};
-          // lane (l32, hsel) holds row l32 of the block, columns 32 j + 8 q + 4 hsel + 0..3
-          char* wrow = turn + (l32 >> 3) * 8192 + (l32 & 7) * 128;
-          const int wkey = (l32 >> 1) & 15;
+          half_t sc[2] = {(half_t)1.f, (half_t)1.f};
+          if (SCALE) scales_of_rows(scale, M, rblock, l16, sc[0], sc[1]);
 #pragma unroll
-          for (int j = 0; j < NB; ++j)
+          for (int hb = 0; hb < 2; ++hb) {
+            const int ib = 2 * i + hb, row = rblock + hb * 16 + l16;
+            if (rblock + hb * 16 >= cur.row_end) continue;
+            if constexpr (SWIGLU) {
+              const half8_t v = swap_halves(swiglu_f16x4(acc[ib][0], acc[ib][2]), swiglu_f16x4(acc[ib][1], acc[ib][3]));
+              const int c0 = cur.n0 + wn * 32 + cofs;
+              if (row < cur.row_end) {
+                half_t* dst = C + (size_t)row * Nout + c0;
+                if (WHOLE) {
+#ifdef GU_NT
+                  __builtin_nontemporal_store(v, reinterpret_cast<half8_t*>(dst));
+#else
+                  *reinterpret_cast<half8_t*>(dst) = v;
+#endif
+                } else {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              const float4_t v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-              half4_t o = __builtin_convertvector(v, half4_t);   // two packed conversions
-              // the product of two fp16 numbers is exact in fp32, so the fp16 multiply rounds as
-              // (half)((float)o * (float)scale) does
-              if (SCALE) o = o * sc4;
-              *reinterpret_cast<half4_t*>(wrow + (((8 * j + 2 * q + hsel) ^ wkey) * 8)) = o;
-            }
-          // piece t holds rows 8 t .. 8 t + 7 of the block; lane = 8 * row + 16-byte part
-          const int rr = lane >> 3, part = lane & 7;
-          const int c0 = cur.n0 + wn * (NB * 32) + 8 * part;
+                  for (int r = 0; r < 8; ++r)
+                    if (c0 + r < Nout) dst[r] = v[r];
+                }
+              }
+            } else {
+              // The wavefront's 64 columns of a row are one 128-byte line, held as two 16-byte pieces
+              // in each of four lanes. Rows n and n + 8 of the unit trade halves (a rotation by 8
+              // inside each row of 16 lanes), so that 8 lanes hold a whole line and a store
+              // instruction writes 8 whole lines: rows 0..7 of the unit, then rows 8..15.
+              half4_t o[WB];
 #pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            const int brow = 8 * t + rr, rkey = (brow >> 1) & 15;
-            half8_t v = *reinterpret_cast<const half8_t*>(turn + t * 8192 + rr * 128 + ((part ^ (rkey >> 1)) * 16));
-            if (rkey & 1) v = __builtin_shufflevector(v, v, 4, 5, 6, 7, 0, 1, 2, 3);   // the XOR swapped the part's two slots
-            const int row = rblock + brow;
-            if (row < cur.row_end) {
-              half_t* dst = C + (size_t)row * Nout + c0;
-              if (WHOLE) {
-                // whole lines that nothing reads again before the launch ends: written through, so
-                // that the caches have less to write back when it does
-                __builtin_nontemporal_store(v, reinterpret_cast<half8_t*>(dst));
-              } else {
+              for (int j = 0; j < WB; ++j) {
+                o[j] = __builtin_convertvector(acc[ib][j], half4_t);   // two packed conversions
+                if (SCALE) {
+                  // the product of two fp16 numbers is exact in fp32, so the fp16 multiply rounds as
+                  // (half)((float)o * (float)scale) does
+                  const half4_t sc4 = {sc[hb], sc[hb], sc[hb], sc[hb]};
+                  o[j] = o[j] * sc4;
+                }
+              }
+              typedef int i4_t __attribute__((ext_vector_type(4)));
+              const i4_t v0 = __builtin_bit_cast(i4_t, swap_halves(o[0], o[1]));   // columns 0..31
+              const i4_t v1 = __builtin_bit_cast(i4_t, swap_halves(o[2], o[3]));   // columns 32..63
+              const bool low = l16 < 8;
+              i4_t got;
 #pragma unroll
-                for (int r = 0; r < 8; ++r)
-                  if (c0 + r < Nout) dst[r] = v[r];
+              for (int d = 0; d < 4; ++d) got[d] = dpp_row_ror<8>(low ? v1[d] : v0[d]);
+              const int c0 = cur.n0 + wn * 64 + (low ? 0 : 32) + cofs;
+#pragma unroll
+              for (int half = 0; half < 2; ++half) {
+                i4_t vi;
+#pragma unroll
+                for (int d = 0; d < 4; ++d) vi[d] = half == 0 ? (low ? v0[d] : got[d]) : (low ? got[d] : v1[d]);
+                const half8_t v = __builtin_bit_cast(half8_t, vi);
+                const int r = rblock + hb * 16 + half * 8 + (l16 & 7);
+                if (r < cur.row_end) {
+                  half_t* dst = C + (size_t)r * Nout + c0;
+                  if (WHOLE) {
+                    // whole lines that nothing reads again before the launch ends: written through,
+                    // so that the caches have less to write back when it does
+                    __builtin_nontemporal_store(v, reinterpret_cast<half8_t*>(dst));
+                  } else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                      if (c0 + e < Nout) dst[e] = v[e];
+                  }
+                }
               }
             }
           }
         }
       };
       if ((Nout & 7) == 0 && cur.n0 + COLS <= Nout) blocks(std::true_type{});
-      else blocks(std::false_type{});
-      // the buffer is the stream's again (the next tile's first iteration fills it): every read
-      // of it has returned by then
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    } else {
-      // ---- epilogue with SwiGLU, 8 bytes of a row per lane (turning the outputs round and holding
-      // the prefetch back, as above, costs the gate/up projection 3 %: 296 us against 287)
-      static_assert(NB == 2, "a wavefront holds gate and up of the same 32 columns");
-      const int chalf = (lane >> 5) * 4;
-      auto blocks = [&](auto whole_columns) {
-        constexpr bool WHOLE = decltype(whole_columns)::value;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int row = cur.row0 + (2 * i + wm) * 32 + l32;
-          if (row >= cur.row_end) continue;
-          half_t* crow = C + (size_t)row * Nout + cur.n0 + wn * 32 + chalf;
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const float4_t g = {acc[i][0][4 * q], acc[i][0][4 * q + 1], acc[i][0][4 * q + 2], acc[i][0][4 * q + 3]};
-            const float4_t u = {acc[i][1][4 * q], acc[i][1][4 * q + 1], acc[i][1][4 * q + 2], acc[i][1][4 * q + 3]};
-            const half4_t o = swiglu_f16x4(g, u);
-            if (WHOLE) {
-              *reinterpret_cast<half4_t*>(crow + 8 * q) = o;
-            } else {
-              const int c0 = cur.n0 + wn * 32 + chalf + 8 * q;
-#pragma unroll
-              for (int r = 0; r < 4; ++r)
-                if (c0 + r < Nout) crow[8 * q + r] = o[r];
-            }
-          }
-        }
-      };
-      if ((Nout & 3) == 0 && cur.n0 + COLS <= Nout) blocks(std::true_type{});
       else blocks(std::false_type{});
     }
     if (!nxt.valid) break;
@@ -864,6 +917,20 @@ int launch_gemm(const half_t* a, const int32_t* a_rows, const half_t* b, const i
 
 }  // namespace
 
+// Rows per tile: 64 while the typical expert fits in one such tile (the launch is then a stream
+// over the weights and the smaller tile halves the padded MFMA work), 128 up to that many, else
+// 256. Under near-uniform routing an expert's rows scatter around the mean by about its square
+// root. Measured on 64 experts, 2048 x 1024: the 256-row tile wins from about 128 rows per
+// expert on. Its loads run three slices ahead, into the next tile, so it wants four slices of
+// K; its tile table is one or two experts per lane.
+int sy_gemm_rows_per_tile(int rows, int E, int K) {
+  const int mean = (rows + E - 1) / E;
+  int typical = mean;
+  while ((typical - mean) * (typical - mean) < 4 * mean) ++typical;
+  const bool stream_ok = K % BIG_BK == 0 && K / BIG_BK >= 4 && E <= 2 * WAVE;
+  return typical <= 64 ? 64 : (typical <= 128 || !stream_ok) ? 128 : 256;
+}
+
 extern "C" SY_API int sy_grouped_gemm(const void* A, const int32_t* a_rows, const void* B, const int32_t* offsets, int E,
                                int rows, int Nout, int K, int swiglu, const void* scale, void* C, void* stream) {
   SY_REQUIRE(rows >= 0 && E >= 1 && Nout >= 1, "grouped_gemm: rows = %d, E = %d, Nout = %d", rows, E, Nout);
@@ -873,21 +940,11 @@ extern "C" SY_API int sy_grouped_gemm(const void* A, const int32_t* a_rows, cons
   SY_REQUIRE(a_rows || (long)rows * K * 2 < (1l << 31), "grouped_gemm: A must stay under 2 GiB (%d rows of %d)", rows, K);
   if (rows == 0) return SY_OK;
   SY_REQUIRE(A && B && offsets && C, "grouped_gemm: null pointer");
-  // rows per tile: 64 while the typical expert fits in one such tile (the launch is then a
-  // stream over the weights and the smaller tile halves the padded MFMA work), else 128. Under
-  // near-uniform routing an expert's rows scatter around the mean by about its square root.
-  const int mean = (rows + E - 1) / E;
-  int typical = mean;
-  while ((typical - mean) * (typical - mean) < 4 * mean) ++typical;
   const half_t* a = (const half_t*)A;
   const half_t* b = (const half_t*)B;
   const half_t* s = (const half_t*)scale;
   half_t* c = (half_t*)C;
-  // measured on 64 experts, 2048 x 1024: the 256-row tile wins from about 128 rows per expert on.
-  // Its loads run three slices ahead, into the next tile, so it wants four slices of K; its tile
-  // table is one or two experts per lane.
-  const bool stream_ok = K % BIG_BK == 0 && K / BIG_BK >= 4 && E <= 2 * WAVE;
-  const int tile = typical <= 64 ? 64 : (typical <= 128 || !stream_ok) ? 128 : 256;
+  const int tile = sy_gemm_rows_per_tile(rows, E, K);
   if (tile == 256 && E <= WAVE) return launch_gemm_stream<1>(a, a_rows, b, offsets, E, rows, Nout, K, swiglu, s, c, (hipStream_t)stream);
   if (tile == 256) return launch_gemm_stream<2>(a, a_rows, b, offsets, E, rows, Nout, K, swiglu, s, c, (hipStream_t)stream);
   if (tile == 64) return launch_gemm<1>(a, a_rows, b, offsets, E, rows, Nout, K, swiglu, s, c, (hipStream_t)stream);
