@@ -7,7 +7,7 @@ namespace sort_core {
 
 constexpr int SORT_THREADS = 1024;
 constexpr int SORT_WAVES = SORT_THREADS / WAVE;  // 16
-constexpr int SMALL_M = 8192;                    // one workgroup sorts up to this many choices
+constexpr int SMALL_M = 2048;                    // one workgroup sorts up to this many choices
 constexpr int PIECE = 512;                       // choices per wavefront in the large path
 constexpr int MAX_E = 512;                     // keeps every launch under 64 KB of LDS
 

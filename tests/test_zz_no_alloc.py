@@ -36,11 +36,11 @@ def test_static_sort_equals_the_workspace_sort_on_two_calls_in_a_row():
 
     ext = kernels.ext()
     lib = ext.lib
-    # both sizes take the launches over many workgroups (more than 8192 choices), which are the
+    # both sizes take the launches over many workgroups (more than 2048 choices), which are the
     # ones that use the histograms; the second call is smaller and finds the first one's there
     for N, E, k, seed in ((40000, 64, 8, 1), (3000, 64, 8, 2), (1500, 128, 8, 3), (100, 64, 8, 4)):
         idx, w = _choices(N, E, k, seed)
-        assert (lib.sy_sort_workspace_bytes(N, k, E) > 0) == (N * k > 8192)
+        assert (lib.sy_sort_workspace_bytes(N, k, E) > 0) == (N * k > 2048)
         rc, got = _static_sort(_abi, lib, idx, w, E)
         assert rc == 0, lib.sy_last_error().decode()
         want = ext.sort_by_expert(idx, w, E)
@@ -61,3 +61,39 @@ def test_static_sort_refuses_what_its_array_cannot_hold():
     idx, w = _choices(N, E, k, 5)
     rc, _ = _static_sort(_abi, lib, idx, w, E)
     assert rc == 1 and "static" in lib.sy_last_error().decode()
+
+
+def test_static_sort_under_stream_capture():
+    """What the entry point is for: after one call outside a capture (which looks the array's
+    address up), a call recorded by a stream capture allocates nothing, so the capture succeeds,
+    and every replay leaves the five outputs of the workspace sort."""
+    from switchyard_amd import _abi, kernels
+
+    ext = kernels.ext()
+    lib = ext.lib
+    N, E, k = 3000, 64, 8
+    idx, w = _choices(N, E, k, 7)
+    rc, _ = _static_sort(_abi, lib, idx, w, E)          # warm-up outside the capture
+    assert rc == 0, lib.sy_last_error().decode()
+    M = N * k
+    i32 = dict(dtype=torch.int32, device=DEV)
+    outs = [torch.full((E,), -1, **i32), torch.full((E + 1,), -1, **i32), torch.full((M,), -1, **i32),
+            torch.zeros(M, dtype=w.dtype, device=DEV), torch.full((M,), -1, **i32)]
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        rc = lib.sy_sort_by_expert_static(idx.data_ptr(), w.data_ptr(), w.element_size(), N, k, E, outs[0].data_ptr(),
+                                          outs[1].data_ptr(), outs[2].data_ptr(), outs[3].data_ptr(), outs[4].data_ptr(),
+                                          _abi._stream())
+    assert rc == 0, lib.sy_last_error().decode()
+    for seed in (8, 9):
+        new_idx, new_w = _choices(N, E, k, seed)
+        idx.copy_(new_idx)
+        w.copy_(new_w)
+        for t in outs:
+            t.fill_(0)
+        graph.replay()
+        torch.cuda.synchronize()
+        want = ext.sort_by_expert(idx, w, E)
+        for name, a, b in zip(("counts", "offsets", "token", "wsorted", "pos_of"), outs, want):
+            assert torch.equal(a, b), (seed, name)
