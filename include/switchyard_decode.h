@@ -67,8 +67,12 @@ SY_API int sy_router_logits(const void* h, const void* router, int N, int H, int
  * choices; outputs (logits included) are bit for bit those of the three separate calls.
  * Limits: those of sy_router_logits, 1 <= N <= 256, E <= 128, 1 <= k <= min(8, E). N == 0 is a
  * no-op. The launch counts its workgroups in a counter of a pool of 1024 that the library keeps
- * in device memory; launches take the counters in turn, so launches on DIFFERENT streams may
- * only disturb each other if one is still waiting to run when the 1024th after it is issued.
+ * in device memory. Launches that run at once take the lower 512 counters in turn, so launches
+ * on DIFFERENT streams may only disturb each other if one is still waiting to run when the 512th
+ * after it is issued. A launch that a stream capture records takes one of the upper 512 in turn
+ * and keeps it for every replay of its graph: no launch outside a capture is ever given that
+ * counter, and two captured launches share one only if 512 launches were captured between them;
+ * graphs that old must not be replayed at the same time as newer ones on another stream.
  * The first call on a device looks the pool's address up (hipGetSymbolAddress): make one call
  * outside stream capture before capturing one. */
 SY_API int sy_router_route_sort(const void* h, const void* router, int N, int H, int E, int k, int norm, void* logits,

@@ -62,8 +62,8 @@ SY_API int sy_sort_by_expert(const int32_t* idx, const void* w, int w_bytes, int
                       size_t workspace_bytes, void* stream);
 
 /* sy_sort_by_expert for callers that cannot allocate (code under HIP graph capture, tight
- * serving loops, harnesses that forbid hipMalloc). It has no counterpart in the reference, whose
- * sort allocates with ATen inside the call (moe_kernels.cu:146-152). Same arguments and results
+ * serving loops, harnesses that forbid hipMalloc). It has no counterpart in the reference: it
+ * exists for those callers only. Same arguments and results
  * as sy_sort_by_expert without the workspace: the per-wavefront histograms live in a static
  * device array of SY_SORT_STATIC_BYTES inside the library (one copy per GPU, held until the
  * process ends). Calls whose sy_sort_workspace_bytes() exceeds that return SY_ERR_ARG (with 64

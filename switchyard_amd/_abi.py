@@ -9,6 +9,7 @@ GIL around every call, as the reference's call guards do.
 
 There is no fallback: if the library is missing and cannot be built, loading raises."""
 
+import collections
 import ctypes
 import threading
 import os
@@ -113,11 +114,12 @@ class Ext:
     """The native module: route, sort_by_expert, grouped_gemv, grouped_gemm, combine."""
 
     PLAN_BYTES_MAX = 32 << 20   # moe_experts keeps the scratch of calls up to this size ...
-    PLANS_MAX = 16              # ... for this many (shape, stream) pairs
+    PLANS_MAX = 16              # ... for this many (shape, stream) pairs, least recently used first out
 
     def __init__(self, lib=None):
         self.lib = lib or load_library()
-        self._plans = {}
+        self._plans = collections.OrderedDict()   # (shape, stream) -> plan; evicted least recently used first
+        self._captured = {}                       # plans that a stream capture has seen: never evicted
         self._plans_lock = threading.Lock()
 
     def _call(self, fn, *args):
@@ -251,36 +253,57 @@ class Ext:
         I, k, norm = down.shape[2], int(k), int(bool(norm))
         stream = _stream()
         # The intermediate results of small calls (a decode step's) live in an allocation that is
-        # kept per shape and stream: calls on one stream run in order, so they may share it.
+        # kept per shape and stream: calls on one stream run in order, so they may share it. A HIP
+        # graph that is captured through this call keeps the allocation's address for as long as it
+        # can be replayed, so a plan that a capture has seen is never evicted; the others leave
+        # least recently used first. (The reference allocates per call, moe_kernels.cu:146-152,272,
+        # 391,438, which costs a call that is waited for the allocator's time in front of its
+        # first launch.)
         key = (N, E, k, H, I, norm, logits is None, bool(one_launch_front), h.device.index, stream)
-        plan = self._plans.get(key)
-        if plan is None:
-            M = N * k
-            need = 0 if one_launch_front else self.lib.sy_sort_workspace_bytes(N, k, E)
-            # idx w counts offsets token wsorted pos_of act y, then the sort's workspace and the logits
-            sizes = [M * 4, M * 2, E * 4, (E + 1) * 4, M * 4, M * 2, M * 4, M * I * 2, M * H * 2, need,
-                     N * E * 2 if logits is None else 0]
-            starts, at = [], 0
-            for size in sizes:
-                starts.append(at)
-                at += (size + 255) // 256 * 256
-            plan = (starts, at, need, None, None)
-            if at <= self.PLAN_BYTES_MAX:
-                if len(self._plans) >= self.PLANS_MAX:
-                    self._plans.pop(next(iter(self._plans)))
-                scratch = torch.empty(at, dtype=torch.uint8, device=h.device)
-                plan = (starts, at, need, scratch, self._addresses(scratch, starts))
-                self._plans[key] = plan
-        starts, at, need, scratch, where = plan
-        if scratch is None:
-            scratch = torch.empty(at, dtype=torch.uint8, device=h.device)
-            return self._enqueue_experts(h, router, logits, gate_up, down, N, H, E, I, k, norm, mfma_tiles, one_launch_front,
-                                         scratch, self._addresses(scratch, starts), need, stream)
-        # kept scratch: two threads enqueueing the same shape on one stream must not interleave
-        # their launches (ctypes releases the GIL inside the calls)
         with self._plans_lock:
-            return self._enqueue_experts(h, router, logits, gate_up, down, N, H, E, I, k, norm, mfma_tiles, one_launch_front,
-                                         scratch, where, need, stream)
+            plan = self._captured.get(key)
+            if plan is None:
+                capturing = torch.cuda.is_current_stream_capturing()
+                plan = self._plans.get(key)
+                if plan is None:
+                    plan = self._new_plan(N, E, k, H, I, logits is None, bool(one_launch_front), h.device)
+                    if plan[3] is not None:
+                        if capturing:
+                            self._captured[key] = plan
+                        else:
+                            if len(self._plans) >= self.PLANS_MAX:
+                                self._plans.popitem(last=False)
+                            self._plans[key] = plan
+                elif capturing:
+                    self._captured[key] = self._plans.pop(key)
+                else:
+                    self._plans.move_to_end(key)
+            starts, at, need, scratch, where = plan
+            if scratch is not None:
+                # kept scratch: two threads enqueueing the same shape on one stream must not
+                # interleave their launches (ctypes releases the GIL inside the calls)
+                return self._enqueue_experts(h, router, logits, gate_up, down, N, H, E, I, k, norm, mfma_tiles,
+                                             one_launch_front, scratch, where, need, stream)
+        scratch = torch.empty(at, dtype=torch.uint8, device=h.device)
+        return self._enqueue_experts(h, router, logits, gate_up, down, N, H, E, I, k, norm, mfma_tiles, one_launch_front,
+                                     scratch, self._addresses(scratch, starts), need, stream)
+
+    def _new_plan(self, N, E, k, H, I, own_logits, one_launch_front, device):
+        """(offsets of the intermediate results, bytes, bytes of the sort's workspace, the kept
+        allocation or None for a call too large to keep one, its addresses)."""
+        M = N * k
+        need = 0 if one_launch_front else self.lib.sy_sort_workspace_bytes(N, k, E)
+        # idx w counts offsets token wsorted pos_of act y, then the sort's workspace and the logits
+        sizes = [M * 4, M * 2, E * 4, (E + 1) * 4, M * 4, M * 2, M * 4, M * I * 2, M * H * 2, need,
+                 N * E * 2 if own_logits else 0]
+        starts, at = [], 0
+        for size in sizes:
+            starts.append(at)
+            at += (size + 255) // 256 * 256
+        if at > self.PLAN_BYTES_MAX:
+            return (starts, at, need, None, None)
+        scratch = torch.empty(at, dtype=torch.uint8, device=device)
+        return (starts, at, need, scratch, self._addresses(scratch, starts))
 
     def experts_routed(self, h, idx, w, gate_up, down, mfma_tiles=False):
         """experts() of the reference in one call of the library: h [N, H], idx int32 [N, k],

@@ -56,7 +56,16 @@ extern "C" SY_API int sy_moe_experts(const void* h, const void* router, void* lo
   // the projections address the gathered rows of h with 32-bit byte offsets
   SY_REQUIRE((long)N * H * 2 < (1l << 31), "moe_experts: h must stay under 2 GiB (%d rows of %d)", N, H);
   int rc;
-  if (router && N > 64) {
+  if (router && N > 64 && !sy_router_route_shape_ok(N, H, E, k)) {
+    // a width the MFMA front does not take (H not a multiple of 512): the row kernel makes the
+    // logits, a workgroup per token, and route and sort are their own launches
+    rc = sy_router_logits(h, router, N, H, E, logits, stream);
+    if (rc) return rc;
+    rc = sy_route(logits, SY_DTYPE_F16, N, E, k, norm, idx, w, stream);
+    if (rc) return rc;
+    rc = sy_sort_by_expert(idx, w, 2, N, k, E, counts, offsets, token, wsorted, pos_of, sort_workspace, sort_workspace_bytes,
+                           stream);
+  } else if (router && N > 64) {
     // beyond the decode kernels' range: one launch for the logits and route, which is also the
     // sort's first pass where the sort runs over many workgroups
     SY_REQUIRE(!one_launch_front, "moe_experts: one_launch_front with a router is for at most 64 tokens");
@@ -133,11 +142,11 @@ extern "C" SY_API int sy_experts_sorted(const void* h, int N, int E, int k, cons
   const int M = N * k;
   // Where it pays, the down projection runs without its row scales: y then holds its rows before
   // the router weight, and the combine multiplies, with the same roundings in the same order.
-  // Fetching the scales costs the weight-stream kernel and the 256-row MFMA tile (which the
-  // GEMM picks from about 108 rows per expert on) more than the multiply costs the combine
-  // (8 tokens: 0.7 us against 0.1; 4096: 3 to 9 us against 0.7); the smaller MFMA tiles gain
-  // nothing, so there the projection scales. `out` has the same bits either way.
-  const bool combine_scales = !mfma_tiles || (long)M >= 108l * E;
+  // Fetching the scales costs the weight-stream kernel and the 256-row MFMA tile more than the
+  // multiply costs the combine (8 tokens: 0.7 us against 0.1; 4096: 3 to 9 us against 0.7); the
+  // smaller MFMA tiles gain nothing, so there the projection scales. `out` has the same bits
+  // either way.
+  const bool combine_scales = !mfma_tiles || sy_gemm_rows_per_tile(M, E, I) == 256;
   const void* scale = combine_scales ? nullptr : wsorted;
   if (mfma_tiles) {
     rc = sy_grouped_gemm(h, token, gate_up, offsets, E, M, I, H, 1, nullptr, act, stream);

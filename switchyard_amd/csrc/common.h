@@ -31,6 +31,10 @@ int sy_sort_assign_counted(const int32_t* idx, const void* w, int N, int k, int 
 int sy_router_route_counting(const void* h, const void* router, int N, int H, int E, int k, int norm, void* logits,
                              int32_t* idx, void* w, void* hist, void* stream);
 bool sy_router_route_counts(int N, int k);
+// front.hip: whether that launch takes the shape (H a multiple of 512, at most 128 experts, top-8)
+bool sy_router_route_shape_ok(int N, int H, int E, int k);
+// gemm.hip: rows of the tile that sy_grouped_gemm picks for `rows` sorted rows over E experts (64, 128 or 256)
+int sy_gemm_rows_per_tile(int rows, int E, int K);
 // decode.hip: router GEMM + route for a few rows (one workgroup per row)
 int sy_router_route_rows(const void* h, const void* router, int N, int H, int E, int k, int norm, void* logits, int32_t* idx,
                          void* w, void* stream);

@@ -715,10 +715,14 @@ namespace {
 constexpr int TICKET_DEVICES = 64;
 std::mutex ticket_mutex;
 unsigned* ticket_base[TICKET_DEVICES] = {nullptr};
-unsigned ticket_next[TICKET_DEVICES] = {0};
+unsigned ticket_next[TICKET_DEVICES][2] = {{0, 0}};
 
-// The counter for the next launch on the current device: slots are handed out in turn.
-int next_ticket(unsigned** out) {
+// The counter for the next launch on the current device. Slots are handed out in turn, the
+// lower half of the pool to launches that run now and the upper half to launches that a stream
+// capture records: a captured launch keeps its slot for every replay of its graph, so no launch
+// outside a capture may ever be given it, and two captured launches share a slot only if half
+// the pool's size in launches was captured between them.
+int next_ticket(unsigned** out, hipStream_t stream) {
   int dev = -1;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= TICKET_DEVICES)
     return sy_fail(SY_ERR_LAUNCH, "router_route_sort: no current device below %d", TICKET_DEVICES);
@@ -730,18 +734,25 @@ int next_ticket(unsigned** out) {
       return sy_fail(SY_ERR_LAUNCH, "router_route_sort: hipGetSymbolAddress: %s", hipGetErrorString(err));
     ticket_base[dev] = static_cast<unsigned*>(p);
   }
-  *out = ticket_base[dev] + ticket_next[dev]++ % front_core::FRONT_TICKETS;
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
+    (void)hipGetLastError();
+    status = hipStreamCaptureStatusNone;
+  }
+  constexpr unsigned HALF = front_core::FRONT_TICKETS / 2;
+  const int captured = status == hipStreamCaptureStatusActive ? 1 : 0;
+  *out = ticket_base[dev] + captured * HALF + ticket_next[dev][captured]++ % HALF;
   return SY_OK;
 }
 
 int front_outputs(const char* what, int N, int E, int k, int norm, int32_t* idx, void* w, int32_t* counts, int32_t* offsets,
-                  int32_t* token, void* wsorted, int32_t* pos_of, front_core::Outputs* out) {
+                  int32_t* token, void* wsorted, int32_t* pos_of, hipStream_t stream, front_core::Outputs* out) {
   SY_REQUIRE(N <= front_core::TAIL_MAX_TOKENS, "%s: at most %d tokens (got %d)", what, front_core::TAIL_MAX_TOKENS, N);
   SY_REQUIRE(E <= 128 && k >= 1 && k <= front_core::TAIL_MAX_K && k <= E, "%s: at most 128 experts and top-8 (got E = %d, k = %d)",
              what, E, k);
   SY_REQUIRE(idx && w && counts && offsets && token && wsorted && pos_of, "%s: null pointer", what);
   unsigned* ticket = nullptr;
-  const int rc = next_ticket(&ticket);
+  const int rc = next_ticket(&ticket, stream);
   if (rc) return rc;
   int nbits = 0;
   while ((1 << nbits) < E) ++nbits;
@@ -758,7 +769,7 @@ extern "C" SY_API int sy_router_route_sort(const void* h, const void* router, in
   if (N == 0) return SY_OK;
   SY_REQUIRE(h && router && logits, "router_route_sort: null pointer");
   front_core::Outputs front;
-  const int rc = front_outputs("router_route_sort", N, E, k, norm, idx, w, counts, offsets, token, wsorted, pos_of, &front);
+  const int rc = front_outputs("router_route_sort", N, E, k, norm, idx, w, counts, offsets, token, wsorted, pos_of, (hipStream_t)stream, &front);
   if (rc) return rc;
   const size_t lds = (size_t)H * sizeof(half_t) + front_core::tail_lds_bytes(N, E, k);
   row_kernel<false, true, FRONT_SORT><<<N, 1024, lds, (hipStream_t)stream>>>(
@@ -794,7 +805,7 @@ extern "C" SY_API int sy_add_rmsnorm_route_sort(const void* x, const void* delta
   if (N == 0) return SY_OK;
   SY_REQUIRE(x && weight && h_out && router && logits, "add_rmsnorm_route_sort: null pointer");
   front_core::Outputs front;
-  const int rc = front_outputs("add_rmsnorm_route_sort", N, E, k, norm, idx, w, counts, offsets, token, wsorted, pos_of, &front);
+  const int rc = front_outputs("add_rmsnorm_route_sort", N, E, k, norm, idx, w, counts, offsets, token, wsorted, pos_of, (hipStream_t)stream, &front);
   if (rc) return rc;
   const size_t lds = (size_t)H * sizeof(half_t) + front_core::tail_lds_bytes(N, E, k);
   row_kernel<false, true, FRONT_SORT><<<N, 1024, lds, (hipStream_t)stream>>>(

@@ -407,6 +407,8 @@ extern "C" SY_API int sy_route_sort(const void* logits, int N, int E, int k, int
 
 // Whether the router + route launch can also be the sort's first pass: the sort runs over many
 // workgroups (above the one-workgroup limit) and a piece is whole groups of 16 tokens.
+bool sy_router_route_shape_ok(int N, int H, int E, int k) { return router_route_shape_ok(N, H, E, k); }
+
 bool sy_router_route_counts(int N, int k) {
   const long M = (long)N * k;
   return M > SMALL_M && piece_for(M) % (RR_TOKENS * k) == 0;

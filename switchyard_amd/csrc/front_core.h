@@ -8,10 +8,11 @@
 // a workgroup that is not last simply ends. The last one puts the counter back to zero, so the
 // next launch that uses it finds it as this one did.
 //
-// The counters are a pool in device memory that the library owns (tickets()); consecutive
-// launches take consecutive slots, so two launches share a slot only if FRONT_TICKETS launches
-// were enqueued between them, and then only matter to each other if they run at the same time
-// on different streams.
+// The counters are a pool in device memory that the library owns; consecutive launches take
+// consecutive slots of one half of the pool (launches recorded by a stream capture of the other
+// half, because they keep their slot for every replay), so two launches share a slot only if
+// FRONT_TICKETS / 2 launches of their kind were enqueued between them, and then only matter to
+// each other if they run at the same time on different streams.
 //
 // Outputs are those of route followed by sort_by_expert of the reference
 // (switchyard/csrc/moe_kernels.cu:73-89,142-157).

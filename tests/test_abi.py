@@ -47,10 +47,14 @@ def test_library_exports_every_declared_symbol(lib):
 
 def test_each_header_citation_names_a_reference_location():
     text = open(HEADER).read()
-    for name in ("sy_route", "sy_sort_by_expert", "sy_sort_by_expert_static", "sy_route_sort", "sy_grouped_gemv", "sy_grouped_gemm", "sy_combine",
+    for name in ("sy_route", "sy_sort_by_expert", "sy_route_sort", "sy_grouped_gemv", "sy_grouped_gemm", "sy_combine",
                  "sy_moe_experts"):
         comment = text[:text.index(f"SY_API int {name}(")].rsplit("/*", 1)[1]
         assert re.search(r"(moe_kernels\.cu|kernels\.py):\d+", comment), name
+    # the entry point that allocates nothing replaces no reference interface and says so
+    comment = text[:text.index("SY_API int sy_sort_by_expert_static(")].rsplit("/*", 1)[1]
+    assert "no counterpart in the reference" in comment and "cannot allocate" in comment
+    assert not re.search(r"(moe_kernels\.cu|kernels\.py):\d+", comment)
 
 
 def test_each_decode_citation_names_a_reference_location():

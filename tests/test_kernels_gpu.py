@@ -207,8 +207,14 @@ def test_grouped_kernels_plain_and_ragged_columns(K, fn, swiglu):
     for e in range(E):
         s, t = int(offsets[e]), int(offsets[e + 1])
         r = F.linear(A[s:t].float(), B[e].float()).cpu()
-        want[s:t] = F.silu(r[:, :Nout]) * r[:, Nout:] if swiglu else r
-    assert (got - want).abs().max().item() < 1e-2
+        # the kernels' rounding points (moe_kernels.cu:253-259,373-378): gate, up, silu(gate) and the
+        # product are each rounded to f16; the plain projection rounds its fp32 sum once
+        want[s:t] = F.silu(r[:, :Nout].half().float()).half().float() * r[:, Nout:].half().float() if swiglu \
+            else r.half().float()
+    assert got.shape == (rows, Nout)
+    # one rounding to f16 of differently ordered fp32 sums: half-precision ulps, and a floor of one
+    # ulp at 1 for outputs near zero
+    assert torch.allclose(got, want, rtol=2.0 ** -9, atol=1e-3)
 
 
 @pytest.mark.parametrize("swiglu", [True, False])
@@ -387,6 +393,27 @@ def test_skewed_routing_is_exact_and_deterministic(K, olmoe, N, kind):
         b = K.experts(h, idx, w, gu, dn, mode)
         assert torch.equal(a, b), "two runs differ"
         assert (a.float() - half.float()).abs().max().item() <= FP16_TOL
+
+
+def test_every_token_on_the_same_eight_experts_at_4096_tokens(K, olmoe):
+    """The most lopsided tile list the MFMA stream can see, through moe_layer: a constant feature
+    in h and a router that weighs it send all 4096 tokens to experts 0..7, so eight experts have
+    4096 rows (16 row tiles each) and 56 have none."""
+    router, gu, dn = olmoe
+    N = 4096
+    h = hidden(N).clone()
+    h[:, 0] = 1.0
+    router = router.clone()
+    router[:, 0] = 0.0
+    router[:8, 0] = 100.0
+    idx, w = K.route(h, router, 8, False)
+    assert torch.bincount(idx.flatten().long(), minlength=64).tolist() == [N] * 8 + [0] * 56
+    a = K.moe_layer(h, router, gu, dn, 8, False)
+    b = K.moe_layer(h, router, gu, dn, 8, False)
+    assert torch.equal(a, b), "two runs differ"
+    half = O.experts_loop(h, idx.long(), w, gu, dn)
+    assert (a.float() - half.float()).abs().max().item() <= FP16_TOL
+    assert torch.equal(K.experts(h, idx, w, gu, dn, "gemm"), a)
 
 
 @pytest.mark.parametrize("N,mode", [(32, "gemv"), (4096, "gemm")])
@@ -569,7 +596,7 @@ def test_router_route_limits(K):
                                        (3000, 64, 8, 128, 64),         # the sort with a workspace
                                        # router GEMM and route in one launch (H a multiple of 512, above 64 tokens):
                                        (100, 64, 8, 512, 128), (300, 128, 8, 512, 64),
-                                       # ... which is also the sort's first pass above 8192 choices
+                                       # ... which is also the sort's first pass above 2048 choices
                                        (1100, 64, 8, 512, 64), (2100, 16, 4, 512, 64), (1027, 60, 8, 1024, 64),
                                        # ... with two and four groups of 16 tokens to a piece of the sort
                                        (9000, 64, 8, 512, 64), (33000, 64, 8, 512, 32)])
@@ -690,3 +717,69 @@ def test_router_route_at_decode_sizes(K, N, E, k, H):
     assert torch.equal(logits, ext.router_logits(h, router))
     ridx, rw = ext.route(logits, k, True)
     assert torch.equal(idx, ridx) and torch.equal(w, rw)
+
+
+def test_moe_experts_entry_point_with_a_width_the_mfma_front_does_not_take(K):
+    """A foreign binding that gives the router for 100 tokens of width 768 (not a multiple of
+    512): the call makes the logits with the row kernel and routes and sorts in launches of
+    their own, with the results of the separate entry points."""
+    N, E, k, H, I = 100, 16, 4, 768, 64
+    h, router, gu, dn = (t.to(DEV) for t in cases.layer(N, E=E, k=k, H=H, I=I, seed=6, wstd=0.05))
+    ext = K.ext()
+    assert not ext.router_route_ok(N, H, E, k)
+    M = N * k
+    i32 = dict(dtype=torch.int32, device=DEV)
+    f16 = dict(dtype=torch.float16, device=DEV)
+    logits, idx, w = torch.empty(N, E, **f16), torch.empty(N, k, **i32), torch.empty(N, k, **f16)
+    counts, offsets = torch.empty(E, **i32), torch.empty(E + 1, **i32)
+    token, wsorted, pos_of = torch.empty(M, **i32), torch.empty(M, **f16), torch.empty(M, **i32)
+    act, y, out = torch.empty(M, I, **f16), torch.empty(M, H, **f16), torch.empty(N, H, **f16)
+    need = ext.lib.sy_sort_workspace_bytes(N, k, E)
+    ws = torch.empty(max(need, 1), dtype=torch.uint8, device=DEV)
+    for tiles in (0, 1):
+        rc = ext.lib.sy_moe_experts(h.data_ptr(), router.data_ptr(), logits.data_ptr(), N, E, k, 0, gu.data_ptr(),
+                                    dn.data_ptr(), H, I, tiles, 0, idx.data_ptr(), w.data_ptr(), counts.data_ptr(),
+                                    offsets.data_ptr(), token.data_ptr(), wsorted.data_ptr(), pos_of.data_ptr(),
+                                    act.data_ptr(), y.data_ptr(), out.data_ptr(), ws.data_ptr(), need,
+                                    torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, ext.lib.sy_last_error()
+        assert torch.equal(logits, ext.router_logits(h, router))
+        ridx, rw = ext.route(logits, k, False)
+        assert torch.equal(idx, ridx) and torch.equal(w, rw)
+        oidx, _ = O.route_logits(logits.cpu(), k, False)
+        assert torch.equal(idx.cpu().long(), oidx)
+        assert torch.equal(out, K.experts(h, ridx, rw, gu, dn, "gemm" if tiles else "gemv"))
+
+
+def test_a_captured_layer_keeps_its_scratch_while_other_shapes_come_and_go(K):
+    """moe_layer keeps the intermediate results of small calls per (shape, stream) and drops the
+    least recently used of them. A HIP graph captured through the call has the allocation's
+    address in its kernel arguments, so that allocation must outlive any number of other shapes:
+    capture a layer of 8 tokens, run more other shapes than the binding keeps, replay."""
+    E, k, H, I = 64, 8, 512, 128
+    _, router, gu, dn = (t.to(DEV) for t in cases.layer(1, E=E, k=k, H=H, I=I, seed=8, wstd=0.05))
+    h = hidden(8, H)
+    ext = K.ext()
+    want = K.moe_layer(h, router, gu, dn, k, False).clone()
+    static_h = h.clone()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = K.moe_layer(static_h, router, gu, dn, k, False)
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(captured, want)
+    kept = len(ext._captured)
+    assert kept >= 1
+    others = []
+    for n in range(9, 9 + ext.PLANS_MAX + 4):     # more shapes than the binding keeps
+        others.append(K.moe_layer(hidden(n, H), router, gu, dn, k, False))
+    big = [torch.empty(32 << 20, dtype=torch.uint8, device=DEV).fill_(0xff) for _ in range(8)]   # reuse freed memory, if any
+    torch.cuda.synchronize()
+    assert len(ext._plans) <= ext.PLANS_MAX and len(ext._captured) == kept
+    for seed in (1, 2):
+        static_h.copy_(hidden(8, H, seed=seed))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(captured, K.moe_layer(static_h, router, gu, dn, k, False))
+    del big, others
