@@ -228,7 +228,10 @@ gemv_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const 
             const int* __restrict__ offsets, int E, int Nout, int K, const half_t* __restrict__ scale,
             half_t* __restrict__ C, int row_cap, SortHere sort = SortHere{}) {
   extern __shared__ __attribute__((aligned(16))) half_t xs[];  // [row_cap][K + ROW_PAD], then the used experts
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  // the wavefront's number is the same in all its lanes, and said so: every unit, K offset and
+  // buffer descriptor below derives from it, and what the compiler cannot prove uniform it wraps
+  // in a loop over the lanes' values, around every load of the stream
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int RS = K + ROW_PAD;
   int* used = reinterpret_cast<int*>(xs + (size_t)row_cap * RS);  // [E] ids of experts with rows, [E] = how many
   const half8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -292,8 +295,11 @@ gemv_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows, const 
     // the part of the range that falls into one expert
     const int u = at / units_per_expert, first = at - u * units_per_expert;
     const int count = min(hi - at, units_per_expert - first);
-    const int e = used[u];
-    const int start = SORT ? s_offsets[e] : offsets[e], end = SORT ? s_offsets[e + 1] : offsets[e + 1];
+    // the same in every lane, and said so: the weights' buffer descriptor is built from it, and a
+    // descriptor that the compiler cannot prove uniform costs every load a loop over its lanes
+    const int e = __builtin_amdgcn_readfirstlane(used[u]);
+    const int start = __builtin_amdgcn_readfirstlane(SORT ? s_offsets[e] : offsets[e]);
+    const int end = __builtin_amdgcn_readfirstlane(SORT ? s_offsets[e + 1] : offsets[e + 1]);
     p.rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(B + (size_t)e * Nfull * K), 0,
                                                (int)((size_t)Nfull * K * 2), 0x00020000);
     // wavefront w takes a contiguous quarter of the units
@@ -371,6 +377,218 @@ int launch_gemv(const void* A, const int32_t* a_rows, const void* B, const int32
   return sy_check_launch("grouped_gemv");
 }
 
+// ---------------------------------------------------------------------------------------------
+// The down projection and combine of a decode step in one launch, for at most 32 sorted rows of
+// at most 4 tokens.
+//
+// With a handful of tokens the combine is a launch's latency around a microsecond of work, and
+// the rows it adds up were written a moment earlier by the launch before it. Here the work is
+// cut by output column instead of by expert: a unit of 4 columns is streamed for every expert
+// that has rows, in ascending expert order, so whoever owns the unit sees all of a token's k
+// rows and can add them up itself, in the order combine adds them, and `y` never exists. Every
+// unit costs the same, so the shares are equal by construction. A workgroup of eight wavefronts
+// takes two units; the four wavefronts of a unit take the experts in turn and leave each row's
+// scaled, rounded values in LDS; after a
+// barrier the rows of every token are added in row order (rows are sorted by expert, so that
+// is ascending expert id, and then by slot, as in combine_kernel). All sorted rows are staged
+// in LDS once, straight from memory, behind the first loads of weights.
+//
+// Measured against the two launches (down projection, then combine; OLMoE shape): 1 token 10.5
+// against 13.9 us, 4 tokens 23 against 26.4; at 8 tokens it loses, 37.0 against 35.2 (every
+// workgroup stages all 64 rows, and a launch cut by column streams at 4.7 TB/s where the one cut
+// by expert reaches 5.7), so it takes up to 4 tokens. Four wavefronts per compute unit with 8, 16
+// or 32 KB in flight each took 41 to 43 us at 8 tokens whatever the depth, and as long with the
+// MFMAs taken out: more wavefronts, not more loads per wavefront, is what a compute unit needs.
+//
+// The roundings are those of the two launches it replaces (gemv_kernel without scales, then
+// combine_kernel<true>): the fp32 dot product in the same K order (a unit starts at the same
+// step of K) rounded to f16, times the router weight rounded to f16, added in fp32.
+constexpr int DC_WAVES = 8, DC_THREADS = DC_WAVES * WAVE;
+constexpr int DC_UNITS = 2;        // units per workgroup; DC_WAVES / DC_UNITS wavefronts share the experts of one
+constexpr int DC_DEPTH = 2;        // chunks of weights (4 KB) a wavefront asks for ahead
+constexpr int DC_MAX_ROWS = 32, DC_MAX_TOKENS = 4, DC_MAX_E = 128;
+
+__host__ __device__ constexpr size_t dc_rows(int M) { return (size_t)(M + 3) / 4 * 4 + 8; }   // staged rows, zero rows behind the last
+__host__ __device__ constexpr size_t dc_lds_bytes(int M, int K, int E) {
+  return dc_rows(M) * (K + ROW_PAD) * sizeof(half_t) + sizeof(float) * 4 * DC_UNITS * DC_MAX_ROWS +
+         sizeof(int) * ((E + 1) + 2 * (DC_MAX_ROWS + 1) + 2 * DC_MAX_ROWS);
+}
+
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"   // m0 carries the LDS address of the staging loads
+template <int NQ>
+__global__ void __launch_bounds__(DC_THREADS)
+gemv_down_combine_kernel(const half_t* __restrict__ act, const half_t* __restrict__ B, const int* __restrict__ offsets,
+                         const int* __restrict__ token, const half_t* __restrict__ wsorted, int E, int Nout, int K, int N,
+                         int M, half_t* __restrict__ out) {
+  constexpr int CH = CH_SHORT;
+  extern __shared__ __attribute__((aligned(16))) half_t xs[];   // [dc_rows(M)][K + ROW_PAD]
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int RS = K + ROW_PAD;
+  const int nrows_lds = (int)dc_rows(M);
+  float* sval = reinterpret_cast<float*>(xs + (size_t)nrows_lds * RS);   // [DC_UNITS][DC_MAX_ROWS][4]
+  int* offs = reinterpret_cast<int*>(sval + 4 * DC_UNITS * DC_MAX_ROWS);   // [E + 1]
+  int* item_e = offs + E + 1;             // [items + 1]: expert of a pass; [DC_MAX_ROWS] = how many
+  int* item_r = item_e + DC_MAX_ROWS + 1;   // first row of the pass
+  int* tok = item_r + DC_MAX_ROWS + 1;    // [M]
+  float* wt = reinterpret_cast<float*>(tok + DC_MAX_ROWS);   // [M]
+
+  // ---- the passes: per expert with rows, ceil(rows / (4 NQ)) of them (one, unless an id repeats)
+  for (int i = tid; i <= E; i += DC_THREADS) offs[i] = offsets[i];
+  for (int i = tid; i < M; i += DC_THREADS) {
+    tok[i] = token[i];
+    wt[i] = (float)wsorted[i];
+  }
+  __syncthreads();
+  if (wave == 0) {
+    int run = 0;
+    for (int e0 = 0; e0 < E; e0 += WAVE) {
+      const int e = e0 + lane;
+      const int n = e < E ? offs[e + 1] - offs[e] : 0;
+      const int mine = (n + 4 * NQ - 1) / (4 * NQ);
+      int inc = mine;
+      for (int o = 1; o < WAVE; o <<= 1) {
+        const int up = __shfl_up(inc, o, WAVE);
+        if (lane >= o) inc += up;
+      }
+      for (int j = 0; j < mine; ++j) {
+        const int at = run + inc - mine + j;
+        if (at < DC_MAX_ROWS) {
+          item_e[at] = e;
+          item_r[at] = offs[e] + j * 4 * NQ;
+        }
+      }
+      run += __shfl(inc, WAVE - 1, WAVE);
+    }
+    if (lane == 0) item_e[DC_MAX_ROWS] = run < DC_MAX_ROWS ? run : DC_MAX_ROWS;
+  }
+  __syncthreads();
+  const int nitems = item_e[DC_MAX_ROWS];
+  const int rows_end = offs[E];
+
+  const int blk = lane >> 2, sub = lane & 3, klane = blk * 8;
+  const int nchunks = K / (CH * STEP_K), nsteps = nchunks * CH;
+  const int units = Nout / UNIT_COLS;
+  constexpr int SHARE = DC_WAVES / DC_UNITS;   // wavefronts per unit
+  const int us = wave / SHARE, part = wave % SHARE;
+  const int mine_items = nitems > part ? (nitems - part + SHARE - 1) / SHARE : 0;
+  const int total = mine_items * nchunks;
+  const size_t bstride = (size_t)Nout * K;
+  // ---- stages every sorted row, straight into LDS (1 KB per instruction: half a row of 1024)
+  const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) char*)xs;
+  auto stage_rows = [&]() {
+    const __amdgpu_buffer_rsrc_t arsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(act), 0, (int)((size_t)M * K * 2), 0x00020000);
+    const int pieces = K / 512;   // 1 KB pieces per row
+    for (int j = wave; j < M * pieces; j += DC_WAVES) {
+      const int r = j / pieces, c = j - r * pieces;
+      const unsigned src = ((unsigned)r * (unsigned)K + (unsigned)c * 512u) * 2u;
+      const unsigned dst = __builtin_amdgcn_readfirstlane(lds_base + (unsigned)(r * RS + c * 512) * 2u);
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                   :: "s"(dst), "v"(src + (unsigned)lane * 16u), "s"(arsrc), "s"(0u) : "memory", "m0");
+    }
+    const half8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int j = tid; j < (nrows_lds - M) * (K / 8); j += DC_THREADS)
+      *reinterpret_cast<half8_t*>(xs + (size_t)(M + j / (K / 8)) * RS + (j % (K / 8)) * 8) = zero8;
+  };
+  bool staged = false;
+
+  for (int ub = blockIdx.x; ub * DC_UNITS < units; ub += gridDim.x) {
+    const int u = ub * DC_UNITS + us;
+    const bool live = u < units;
+    const int rot = (u * 5) % nsteps;
+    const unsigned lane_off = (((unsigned)(u * UNIT_COLS + sub)) * (unsigned)K + (unsigned)klane) * 2u;
+    Chunk<CH> buf[DC_DEPTH];
+    auto issue = [&](Chunk<CH>& c, int i) {
+      const int it = i / nchunks, ch = i - it * nchunks;
+      const int e = __builtin_amdgcn_readfirstlane(item_e[part + it * SHARE]);
+      const __amdgpu_buffer_rsrc_t rsrc =
+          __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(B + (size_t)e * bstride), 0, (int)(bstride * 2), 0x00020000);
+#pragma unroll
+      for (int s = 0; s < CH; ++s) {
+        const int at = ch * CH + s + rot;
+        const int kk = (at - (at >= nsteps ? nsteps : 0)) * STEP_K;
+        c.w[s] = load_stream(rsrc, lane_off, (unsigned)kk * 2u);
+      }
+    };
+    float4_t acc[NQ];
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) acc[q] = float4_t{0.f, 0.f, 0.f, 0.f};
+    auto compute = [&](const Chunk<CH>& c, int i) {
+      const int it = i / nchunks, ch = i - it * nchunks;
+      const int r0 = __builtin_amdgcn_readfirstlane(item_r[part + it * SHARE]);
+      const half_t* xlane = xs + (size_t)(r0 + sub) * RS + klane;
+#pragma unroll
+      for (int s = 0; s < CH; ++s) {
+        const int at = ch * CH + s + rot;
+        const int kk = (at - (at >= nsteps ? nsteps : 0)) * STEP_K;
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) {
+          const half8_t x = *reinterpret_cast<const half8_t*>(xlane + q * QUAD * RS + kk);
+          acc[q] = __builtin_amdgcn_mfma_f32_4x4x4f16(lo4(c.w[s]), lo4(x), acc[q], 0, 0, 0);
+          acc[q] = __builtin_amdgcn_mfma_f32_4x4x4f16(hi4(c.w[s]), hi4(x), acc[q], 0, 0, 0);
+        }
+      }
+      if (ch != nchunks - 1) return;
+      // the pass is through K: sum the 16 K-slices; lane j < 4 then holds the unit's 4 columns of row r0 + 4q + j
+      const int e = __builtin_amdgcn_readfirstlane(item_e[part + it * SHARE]);
+      const int last = min(__builtin_amdgcn_readfirstlane(offs[e + 1]), r0 + 4 * NQ);
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) {
+        float4_t v;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = sum_blocks(acc[q][j]);
+        acc[q] = float4_t{0.f, 0.f, 0.f, 0.f};
+        const int r = r0 + q * QUAD + lane;
+        if (lane < QUAD && r < last) {
+          const float scale = wt[r];
+          float4_t o;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) o[j] = (float)(half_t)((float)(half_t)v[j] * scale);
+          *reinterpret_cast<float4_t*>(sval + ((size_t)us * DC_MAX_ROWS + r) * 4) = o;
+        }
+      }
+    };
+    if (live) {
+#pragma unroll
+      for (int b = 0; b < DC_DEPTH; ++b)
+        if (b < total) issue(buf[b], b);
+    }
+    if (!staged) {
+      // The sorted rows go into LDS behind the first loads of weights, so that the two latencies
+      // overlap; vmcnt(0) because the compiler does not know of these loads (the weights asked
+      // for above are older and have landed by then too).
+      stage_rows();
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      staged = true;
+    }
+    if (live) {
+      for (int i0 = 0; i0 < total; i0 += DC_DEPTH) {
+#pragma unroll
+        for (int b = 0; b < DC_DEPTH; ++b) {
+          const int i = i0 + b;
+          if (i < total) {
+            compute(buf[b], i);
+            if (i + DC_DEPTH < total) issue(buf[b], i + DC_DEPTH);
+          }
+        }
+      }
+    }
+    __syncthreads();
+    // ---- combine: thread (unit, token, column) adds the token's rows in row order
+    if (tid < DC_UNITS * N * 4) {
+      const int cu = tid / (N * 4), t = (tid / 4) % N, j = tid & 3;
+      const int col = (ub * DC_UNITS + cu) * UNIT_COLS + j;
+      float sum = 0.f;
+      for (int r = 0; r < rows_end; ++r)
+        if (tok[r] == t) sum += sval[((size_t)cu * DC_MAX_ROWS + r) * 4 + j];
+      if (col < Nout) out[(size_t)t * Nout + col] = (half_t)sum;
+    }
+    __syncthreads();
+  }
+}
+#pragma clang diagnostic pop
+
 }  // namespace
 
 // The gate/up projection (SwiGLU) of a decode step straight from the routing: sort_by_expert of
@@ -387,6 +605,36 @@ int sy_grouped_gemv_sorting(const void* h, const int32_t* idx, const void* w, in
   while ((1 << nbits) < E) ++nbits;
   const SortHere sort{idx, (const half_t*)w, N * k, k, nbits, counts, offsets, token, (half_t*)wsorted, pos_of};
   return launch_gemv(h, nullptr, gate_up, nullptr, E, N * k, N, I, H, 1, nullptr, act, (hipStream_t)stream, &sort);
+}
+
+// Whether sy_gemv_down_combine takes this shape.
+bool sy_gemv_combines(int N, int k, int E, int H, int I) {
+  const long M = (long)N * k;
+  return N >= 1 && N <= DC_MAX_TOKENS && k >= 1 && M <= DC_MAX_ROWS && E >= 1 && E <= DC_MAX_E && I % (CH_SHORT * STEP_K) == 0 &&
+         I >= CH_SHORT * STEP_K && H % UNIT_COLS == 0 && H >= UNIT_COLS && dc_lds_bytes((int)M, I, E) <= 160 * 1024 &&
+         (long)H * I * 2 < (1l << 31);
+}
+
+// The down projection and combine of a decode step in one launch: act f16 [M, I] sorted rows,
+// down f16 [E, H, I], the sort's offsets / token / wsorted -> out f16 [N, H], with the bits of
+// sy_grouped_gemv (no scale) followed by the combine that applies the router weights.
+int sy_gemv_down_combine(const void* act, const void* down, const int32_t* offsets, const int32_t* token, const void* wsorted,
+                         int N, int k, int E, int H, int I, void* out, void* stream) {
+  SY_REQUIRE(sy_gemv_combines(N, k, E, H, I), "gemv_down_combine: N = %d, k = %d, E = %d, H = %d, I = %d", N, k, E, H, I);
+  SY_REQUIRE(act && down && offsets && token && wsorted && out, "gemv_down_combine: null pointer");
+  const int M = N * k;
+  const size_t lds = dc_lds_bytes(M, I, E);
+  const int units = H / UNIT_COLS;
+  int grid = (units + DC_UNITS - 1) / DC_UNITS;
+  const int cus = sy_compute_units();
+  grid = grid > cus ? cus : grid;
+  void (*kern)(const half_t*, const half_t*, const int*, const int*, const half_t*, int, int, int, int, int, half_t*) =
+      gemv_down_combine_kernel<1>;   // at most 4 tokens: one quad of rows per expert (more only if an id repeats)
+  if (lds > 48 * 1024 && hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+    return sy_fail(SY_ERR_LAUNCH, "gemv_down_combine: cannot reserve %zu bytes of LDS", lds);
+  kern<<<grid, DC_THREADS, lds, (hipStream_t)stream>>>((const half_t*)act, (const half_t*)down, offsets, token,
+                                                      (const half_t*)wsorted, E, H, I, N, M, (half_t*)out);
+  return sy_check_launch("gemv_down_combine");
 }
 
 // Whether sy_grouped_gemv_sorting takes this shape: one choice per lane of a wavefront.
