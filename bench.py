@@ -184,7 +184,16 @@ def layer_record(kernels, N, layers, mode, steps, warmup):
     flops = N * TOPK * 6 * H * I
     gbs, gbs_ev = used_mean * EXPERT_BYTES / ms_stream / 1e6, used[0] * EXPERT_BYTES / ms_event / 1e6
     tf = flops / ms_stream / 1e9
+    # the bytes a layer must move: the used experts' weights once, and per sorted row the gathered
+    # row of h, act written and read, y written and read: M * (3 H + 2 I) * 2 B = M * 16 384 B here
+    layer_bytes = used_mean * EXPERT_BYTES + N * TOPK * (3 * H + 2 * I) * 2
+    by_bytes = {"bound": "hbm", "achieved": layer_bytes / ms_stream / 1e6, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": layer_bytes / ms_stream / 1e6 / HBM_PEAK_GBS, "traffic": measured_traffic(N, "layer"),
+                "kernel": "whole layer (front, sort, two projections, combine)", "us_per_launch": ms_stream * 1e3,
+                "algorithmic_per_launch": layer_bytes,
+                "bytes": "used experts' weights + N*k*(3H + 2I)*2 B of activations (gathered h rows, act and y written and read)"}
     return {"tokens": N, "mode": mode if mode != "auto" else kernels._auto(N, N * TOPK, E), "us_per_layer": ms_stream * 1e3,
+            "roofline_bytes": by_bytes,
             "us_per_layer_event_median": ms_event * 1e3, "experts_used_mean": used_mean, "experts_used_layer0": used[0],
             "weight_GBps": gbs, "weight_GBps_event_median": gbs_ev, "frac_of_hbm_peak": gbs / HBM_PEAK_GBS,
             "frac_of_hbm_peak_event_median": gbs_ev / HBM_PEAK_GBS, "tflops": tf,
@@ -193,32 +202,42 @@ def layer_record(kernels, N, layers, mode, steps, warmup):
 
 
 def projection_times(kernels, N, layers, mode, reps, warmup):
-    """The two grouped projections of the layer, each timed per launch in a stream of launches
-    of that kernel alone (events on the launch stream), rotating through the layers' weights.
-    Returns (gate/up ms, down ms, used experts per layer, whether the weight-stream kernel ran)."""
+    """The two grouped projections as the layer launches them, each timed per launch in a stream
+    of launches of that kernel alone (events on the launch stream), rotating through the layers'
+    weights. Returns (gate/up ms, down ms, used experts per layer, names of the two kernels).
+    What moe_layer launches: on the weight-stream path up to 64 choices the gate/up stream that
+    sorts the choices itself (sy_grouped_gemv_sorting) and a down projection without row scales
+    (the combine applies the router weights); on the MFMA tiles sy_grouped_gemm, the down
+    projection without row scales where the 256-row tile runs, with them on the smaller tiles."""
     dev = "cuda:0"
     h = hidden(N).to(dev)
     M = N * TOPK
     use_gemv = (mode if mode != "auto" else kernels._auto(N, M, E)) == "gemv"
+    X = kernels.ext()
+    sorting = use_gemv and M <= 64
+    big_tile = not use_gemv and M >= 108 * E           # sy_gemm_rows_per_tile(M, E, K) == 256 for these shapes
+    down_scaled = not use_gemv and not big_tile
     rot, used = [], []
     for router, gu, dn in layers:
         idx, w = routed_ids(kernels, h, router)
-        counts, offsets, token, wsorted, pos_of = kernels.ext().sort_by_expert(idx, w, E)
+        counts, offsets, token, wsorted, pos_of = X.sort_by_expert(idx, w, E)
         used.append(int((counts > 0).sum()))
-        rot.append((gu, dn, offsets, token, wsorted))
+        rot.append((gu, dn, offsets, token, wsorted, idx, w))
     act = torch.randn(M, I, generator=torch.Generator().manual_seed(7)).mul_(0.3).half().to(dev)
     calls = [0]
-    X = kernels.ext()
 
     def gate_up():
-        gu, _, off, tok, _ = rot[calls[0] % len(rot)]
+        gu, _, off, tok, _, idx, w = rot[calls[0] % len(rot)]
         calls[0] += 1
+        if sorting:
+            return X.grouped_gemv_sorting(h, idx, w, gu)
         return X.grouped_gemv(h, tok, gu, off, M, True, None, N) if use_gemv else X.grouped_gemm(h, tok, gu, off, None, 0, M, True, None)
 
     def down():
-        _, dn, off, _, ws = rot[calls[0] % len(rot)]
+        _, dn, off, _, ws, _, _ = rot[calls[0] % len(rot)]
         calls[0] += 1
-        return X.grouped_gemv(act, None, dn, off, M, False, ws, N) if use_gemv else X.grouped_gemm(act, None, dn, off, None, 0, M, False, ws)
+        scale = ws if down_scaled else None
+        return X.grouped_gemv(act, None, dn, off, M, False, scale, N) if use_gemv else X.grouped_gemm(act, None, dn, off, None, 0, M, False, scale)
 
     out = []
     for fn in (gate_up, down):
@@ -228,19 +247,30 @@ def projection_times(kernels, N, layers, mode, reps, warmup):
         calls[0] = 0
         t = stream_times(fn, max(reps, 20), 10)
         out.append(sum(t) / len(t))
-    return out[0], out[1], used, use_gemv
+    if use_gemv:
+        names = ("gemv_kernel<swiglu, sorts its choices> (gate/up projection, sy_grouped_gemv_sorting)" if sorting
+                 else "gemv_kernel<swiglu> (gate/up projection)",
+                 "gemv_kernel<no row scales> (down projection; the combine applies the router weights)"
+                 + (" [up to 4 tokens the layer runs gemv_down_combine_kernel instead: down projection and combine in one launch]"
+                    if N <= 4 else ""))
+    else:
+        tile = "gemm_stream_kernel, 256-row tile" if big_tile else "gemm_kernel, 64/128-row tile"
+        names = (f"{tile} <swiglu> (gate/up projection)",
+                 f"{tile} <{'row scales' if down_scaled else 'no row scales'}> (down projection"
+                 + ("" if down_scaled else "; combine_kernel<weighted> applies the router weights") + ")")
+    return out[0], out[1], used, use_gemv, names
 
 
 def projection_rooflines(kernels, N, layers, mode, reps, warmup):
     """`roofline` objects of the gate/up projection (the dominant kernel) and of the down
-    projection at N tokens. Bound and algorithmic figure: below about 300 rows per expert the
+    projection at N tokens, for the kernels the layer launches. Bound and algorithmic figure: below about 300 rows per expert the
     launch is a stream over the used experts' weights (bytes, against HBM peak), above it is
     bound by the MFMAs (flops, against dense fp16 peak)."""
-    gu_ms, dn_ms, used, use_gemv = projection_times(kernels, N, layers, mode, reps, warmup)
+    gu_ms, dn_ms, used, use_gemv, names = projection_times(kernels, N, layers, mode, reps, warmup)
     used_mean = sum(used) / len(used)
     M = N * TOPK
     out = []
-    for name, ms, share, src in (("gate/up", gu_ms, 2, "gate_up"), ("down", dn_ms, 1, "down")):
+    for name, ms, share, src in ((names[0], gu_ms, 2, "gate_up"), (names[1], dn_ms, 1, "down")):
         if use_gemv or M // E < 300:
             alg = used_mean * share * H * I * 2
             roof = {"bound": "hbm", "achieved": alg / ms / 1e6, "peak": HBM_PEAK_GBS, "unit": "GB/s"}
@@ -249,8 +279,7 @@ def projection_rooflines(kernels, N, layers, mode, reps, warmup):
             roof = {"bound": "mfma", "achieved": alg / ms / 1e9, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s"}
         roof["frac"] = roof["achieved"] / roof["peak"]
         roof["traffic"] = measured_traffic(N, ("gemv_" if use_gemv else "gemm_") + src)
-        epi = "swiglu" if share == 2 else "scale"
-        roof["kernel"] = f"{'gemv_kernel' if use_gemv else 'grouped_gemm'}<{epi}> ({name} projection)"
+        roof["kernel"] = name
         roof["us_per_launch"] = ms * 1e3
         roof["algorithmic_per_launch"] = alg
         out.append(roof)
@@ -286,11 +315,16 @@ def library_batched_gemm(layers, N, reps=50):
     return out
 
 
-def cpu_loop_baseline(h, router, gu, dn, used, reps=5):
-    """The reference per-expert loop (switchyard/moe.py:34-42) restated in oracle/, fp32, on the host."""
+def cpu_loop_baseline(h, router, gu, dn, used, reps=5, weights32=None, dtype=torch.float32):
+    """The reference per-expert loop (switchyard/moe.py:34-42) restated in oracle/, on the host,
+    fp32 (or fp16: weights and activations as the GPU has them), median of `reps` after 1 warm-up."""
     from oracle import moe_oracle as O
 
-    hf, rf, gf, df = h.float(), router.float(), gu.float(), dn.float()
+    if dtype == torch.float32:
+        rf, gf, df = weights32 if weights32 is not None else (router.float(), gu.float(), dn.float())
+        hf = h.float()
+    else:
+        hf, rf, gf, df = h, router, gu, dn
     idx, w = O.route(hf, rf, TOPK, False)
     O.experts_loop(hf, idx, w, gf, df)
     times = []
@@ -299,15 +333,36 @@ def cpu_loop_baseline(h, router, gu, dn, used, reps=5):
         O.experts_loop(hf, idx, w, gf, df)
         times.append(time.perf_counter() - t0)
     t = statistics.median(times)
+    name = "fp32" if dtype == torch.float32 else "fp16"
     return {"value": used * EXPERT_BYTES / t / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"oracle per-expert loop, fp32 weights, {h.shape[0]} tokens, median of {reps} passes "
+            "sample": f"oracle per-expert loop, {name} weights, {h.shape[0]} tokens, median of {reps} passes "
                       f"({t * 1e3:.1f} ms each) after 1 warm-up; os.cpu_count()={os.cpu_count()}",
-            "us_per_layer": t * 1e6}
+            "us_per_layer": t * 1e6, "tokens": h.shape[0], "dtype": name,
+            "tflops": h.shape[0] * TOPK * 6 * H * I / t / 1e12}
 
 
-def gpu_loop_baseline(layers, sizes=(8, 4096)):
-    """The reference's "loop" column (bench/kernels.py:41): the same per-expert PyTorch loop in fp16
-    on the GPU, event-timed like the kernels (median of 5 after 1 warm-up), ms per layer."""
+def cpu_baselines(cpu_layer, sizes, fp16_up_to=32):
+    """The CPU loop at every token count of the metric: fp32 weights for all of them (median of 5,
+    3 at 4096 tokens), fp16 too up to 32 tokens; the thread count is in every record."""
+    from oracle import moe_oracle as O
+
+    router, gu, dn = cpu_layer
+    w32 = (router.float(), gu.float(), dn.float())
+    out = {}
+    for N in sizes:
+        h = hidden(N)
+        idx, _ = O.route(h.float(), w32[0], TOPK, False)
+        used = int((torch.bincount(idx.flatten(), minlength=E) > 0).sum())
+        out[str(N)] = cpu_loop_baseline(h, router, gu, dn, used, reps=3 if N >= 4096 else 5, weights32=w32)
+        if N <= fp16_up_to:
+            out[f"{N}_fp16"] = cpu_loop_baseline(h, router, gu, dn, used, reps=3, dtype=torch.float16)
+    return out
+
+
+def gpu_loop_baseline(layers, sizes=(1, 8, 32, 256, 1024, 4096)):
+    """The reference's "loop" and "sorted loop" columns (bench/kernels.py:41-42): the per-expert
+    PyTorch loop and the loop over sorted rows, in fp16 on the GPU, event-timed like the kernels
+    (median of 5 after 1 warm-up), ms per layer."""
     from oracle import moe_oracle as O
 
     router, gu, dn = layers[0]
@@ -316,8 +371,10 @@ def gpu_loop_baseline(layers, sizes=(8, 4096)):
         h = hidden(N).to("cuda:0")
         idx, w = O.route(h, router, TOPK, False)
         O.experts_loop(h, idx, w, gu, dn)
+        O.experts_grouped(h, idx, w, gu, dn)
         torch.cuda.synchronize()
-        out[str(N)] = {"ms_per_layer": statistics.median(event_times(lambda: O.experts_loop(h, idx, w, gu, dn), 5))}
+        out[str(N)] = {"ms_per_layer": statistics.median(event_times(lambda: O.experts_loop(h, idx, w, gu, dn), 5)),
+                       "sorted_loop_ms_per_layer": statistics.median(event_times(lambda: O.experts_grouped(h, idx, w, gu, dn), 5))}
     return out
 
 
@@ -351,8 +408,11 @@ def decode_rates(batches=(8, 64), prompt_len=512, new_tokens=128):
     head_bytes = s.vocab * s.hidden * 2
     router_bytes = s.layers * s.experts * s.hidden * 2
     out = {"model": "OLMoE-1B-7B shape, 16 layers, random-init fp16", "prompt_len": prompt_len,
-           "new_tokens": new_tokens, "step": "HIP-graph replay of Decoder.step_fused (every launch a kernel of this library)",
-           "as_written_step": "HIP-graph replay of Decoder.step_static: attention in PyTorch operators, MoE through the hook",
+           "new_tokens": new_tokens,
+           "step": "the configuration as written: attention in PyTorch operators, the MoE layers through the hook -> "
+                   "kernels.moe_layer (HIP-graph replay of Decoder.step_static)",
+           "fused_step": "beside it, not the stated configuration: HIP-graph replay of Decoder.step_fused, in which the "
+                         "attention side runs on this library's kernels too",
            "bytes_per_step": "used experts' weights of 16 layers + attention, router and lm_head weights + the KV cache "
                              "at the mean length of the run; roofline_frac = bytes / 8 TB/s / step time"}
     for B in batches:
@@ -388,19 +448,22 @@ def decode_rates(batches=(8, 64), prompt_len=512, new_tokens=128):
         ref_first = loop_model.forward(tokens)[:, -1]
         agree = first.argmax(-1) == ref_first.argmax(-1)
         agree_w = first_w.argmax(-1) == ref_first.argmax(-1)
-        out[f"b{B}"] = {"tok_per_s": B / step_s, "ms_per_step": step_s * 1e3,
-                        "prefill_tok_per_s": B * prompt_len / tm["prefill_s"],
-                        "attention_torch_tok_per_s": B * tw["decode_steps"] / tw["decode_s"],
-                        "attention_torch_ms_per_step": tw["decode_s"] * 1e3 / tw["decode_steps"],
+        written_s = tw["decode_s"] / tw["decode_steps"]
+        out[f"b{B}"] = {"tok_per_s": B / written_s, "ms_per_step": written_s * 1e3,
+                        "prefill_tok_per_s": B * prompt_len / tw["prefill_s"],
                         "experts_used_per_layer_mean": sum(used) / len(used), "bytes_per_step": step_bytes,
                         "roofline_tok_per_s": B * HBM_PEAK_GBS * 1e9 / step_bytes,
-                        "roofline_frac": step_bytes / (HBM_PEAK_GBS * 1e9) / step_s,
-                        "attention_torch_roofline_frac": step_bytes / (HBM_PEAK_GBS * 1e9) / (tw["decode_s"] / tw["decode_steps"]),
-                        "moe_ms_per_step": moe_ms * s.layers, "moe_share_of_step": moe_ms * s.layers / (step_s * 1e3),
-                        "moe_share_of_attention_torch_step": moe_ms * s.layers / (tw["decode_s"] * 1e3 / tw["decode_steps"]),
-                        "top1_rows_identical_to_loop_hook": int(agree.sum()),
-                        "attention_torch_top1_rows_identical_to_loop_hook": int(agree_w.sum()), "rows": B,
-                        "first_logits_max_abs_diff_vs_loop_hook": (first.float() - ref_first.float()).abs().max().item()}
+                        "roofline_frac": step_bytes / (HBM_PEAK_GBS * 1e9) / written_s,
+                        "moe_ms_per_step": moe_ms * s.layers, "moe_share_of_step": moe_ms * s.layers / (written_s * 1e3),
+                        "top1_rows_identical_to_loop_hook": int(agree_w.sum()), "rows": B,
+                        "first_logits_max_abs_diff_vs_loop_hook": (first_w.float() - ref_first.float()).abs().max().item(),
+                        "fused_step": {"tok_per_s": B / step_s, "ms_per_step": step_s * 1e3,
+                                       "prefill_tok_per_s": B * prompt_len / tm["prefill_s"],
+                                       "roofline_frac": step_bytes / (HBM_PEAK_GBS * 1e9) / step_s,
+                                       "moe_share_of_step": moe_ms * s.layers / (step_s * 1e3),
+                                       "top1_rows_identical_to_loop_hook": int(agree.sum()),
+                                       "first_logits_max_abs_diff_vs_loop_hook":
+                                           (first.float() - ref_first.float()).abs().max().item()}}
     return out
 
 
@@ -432,7 +495,12 @@ def run_default(args):
     roof, roof_down = projection_rooflines(kernels, N, layers, mode, args.steps, args.warmup)
 
     whole = not args.no_cpu and N == 8 and mode == "auto"   # the default run reports the whole metric
-    cpu = None if args.no_cpu else cpu_loop_baseline(h_cpu, *cpu_layers[0], used[0])
+    cpu = cpu_sizes = None
+    if whole:
+        cpu_sizes = cpu_baselines(cpu_layers[0], sorted(set(DECODE_SIZES + PREFILL_SIZES)))
+        cpu = cpu_sizes[str(N)]
+    elif not args.no_cpu:
+        cpu = cpu_loop_baseline(h_cpu, *cpu_layers[0], used[0])
     sizes = prefill = gpu_loop = decode = None
     if whole:
         sizes = {str(n): layer_record(kernels, n, layers, "auto", 100, 10) for n in DECODE_SIZES}
@@ -447,6 +515,8 @@ def run_default(args):
         except Exception as exc:  # a comparison, not part of the metric
             prefill["library_batched_gemm_even_routing"] = {"error": f"{type(exc).__name__}: {exc}"}
         prefill["other_sizes"] = {str(n): layer_record(kernels, n, layers, "gemm", 50, 5) for n in PREFILL_SIZES if n != big}
+        for rec in prefill["other_sizes"].values():   # these sizes are bound by the bytes the layer moves, not by the MFMAs
+            rec["roofline"] = rec.pop("roofline_bytes")
         gpu_loop = gpu_loop_baseline(layers)
         n_layers = len(layers)
         del layers
@@ -475,7 +545,8 @@ def run_default(args):
         "vs_baseline_note": "published figure is the reference's on one Tesla T4 (320 GB/s), event-timed single calls; "
                             "`value` is the stream-of-layers figure, `value_event_median` the like-for-like one",
         "gpu": torch.cuda.get_device_name(0),
-        "roofline": roof, "down_projection": roof_down, "cpu_baseline": cpu, "gpu_loop_fp16": gpu_loop,
+        "roofline": roof, "down_projection": roof_down, "cpu_baseline": cpu, "cpu_baseline_sizes": cpu_sizes,
+        "gpu_loop_fp16": gpu_loop,
         "decode_sizes": sizes, "prefill": prefill, "decode": decode,
     }
     print(json.dumps(line), flush=True)

@@ -109,6 +109,19 @@ SY_API int sy_route_sort(const void* logits, int N, int E, int k, int norm, int3
 SY_API int sy_grouped_gemv(const void* A, const int32_t* a_rows, const void* B, const int32_t* offsets, int E, int rows,
                            int max_rows_hint, int Nout, int K, int swiglu, const void* scale, void* C, void* stream);
 
+/* sort_by_expert() and the gate/up grouped_gemv() of a decode step in ONE launch: replaces the two
+ * calls as experts() makes them (switchyard/kernels.py:84,67; moe_kernels.cu:142-157,385-415) for
+ * at most 64 choices. Every workgroup of the weight stream sorts the choices itself (one per lane
+ * of a wavefront) where it would otherwise read `offsets`, and the first one also writes the
+ * sort's five results for the launches behind it. h f16 [N,H]; idx int32 [N,k]; w f16 [N,k];
+ * gate_up f16 [E,2I,H] -> counts, offsets, token, wsorted, pos_of as sy_sort_by_expert leaves
+ * them and act f16 [N*k, I] as sy_grouped_gemv (swiglu) does, bit for bit. This is the gate/up
+ * launch of sy_moe_experts / sy_experts_routed at decode.
+ * Limits: N*k <= 64, E <= 128, k <= E, H % 8 == 0, H <= 4096. */
+SY_API int sy_grouped_gemv_sorting(const void* h, const int32_t* idx, const void* w, int N, int k, const void* gate_up,
+                                   int E, int I, int H, int32_t* counts, int32_t* offsets, int32_t* token,
+                                   void* wsorted, int32_t* pos_of, void* act, void* stream);
+
 /* Replaces grouped_gemm() (moe_kernels.cu:264-298, kernel :167-261): the same function on
  * MFMA tiles for many rows per expert. The row tiles of every expert are derived from
  * `offsets` inside the kernel, so the reference's tile_offsets / total_tiles arguments (and

@@ -35,6 +35,8 @@ SIGNATURES = {
                                _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
     "sy_grouped_gemv": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int,
                                  _c_int, _c_void_p, _c_void_p, _c_void_p]),
+    "sy_grouped_gemv_sorting": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_int]
+                                + [_c_void_p] * 7),
     "sy_grouped_gemm": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int,
                                  _c_void_p, _c_void_p, _c_void_p]),
     "sy_combine": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p]),
@@ -207,6 +209,27 @@ class Ext:
         """max_rows: an upper bound on the rows of one expert if known (0: unknown); a sizing
         hint with no effect on the result."""
         return self._grouped(self.lib.sy_grouped_gemv, A, a_rows, B, offsets, rows, swiglu, scale, hint=max_rows)
+
+    def grouped_gemv_sorting(self, h, idx, w, gate_up):
+        """sort_by_expert and the gate/up weight stream of a decode step in one launch (at most 64
+        choices): h [N, H], idx int32 [N, k], w f16 [N, k], gate_up [E, 2I, H] ->
+        [counts, offsets, token, wsorted, pos_of, act [N*k, I]]."""
+        for t, name, dt in ((h, "h", torch.float16), (idx, "idx", torch.int32), (w, "w", torch.float16),
+                            (gate_up, "gate_up", torch.float16)):
+            _check(t, name, dt)
+        (N, H), k, E = h.shape, idx.shape[1], gate_up.shape[0]
+        I, M, dev = gate_up.shape[1] // 2, N * k, h.device
+        if tuple(idx.shape) != (N, k) or tuple(w.shape) != (N, k) or gate_up.shape[2] != H:
+            raise RuntimeError("grouped_gemv_sorting: idx and w must be [N, k], gate_up [E, 2I, H]")
+        i32 = dict(dtype=torch.int32, device=dev)
+        counts, offsets = torch.empty(E, **i32), torch.empty(E + 1, **i32)
+        token, pos_of = torch.empty(M, **i32), torch.empty(M, **i32)
+        wsorted = torch.empty(M, dtype=torch.float16, device=dev)
+        act = torch.empty((M, I), dtype=torch.float16, device=dev)
+        self._call(self.lib.sy_grouped_gemv_sorting, h.data_ptr(), idx.data_ptr(), w.data_ptr(), N, k, gate_up.data_ptr(),
+                   E, I, H, counts.data_ptr(), offsets.data_ptr(), token.data_ptr(), wsorted.data_ptr(), pos_of.data_ptr(),
+                   act.data_ptr(), _stream())
+        return [counts, offsets, token, wsorted, pos_of, act]
 
     def grouped_gemm(self, A, a_rows, B, offsets, tile_offsets, total_tiles, rows, swiglu, scale):
         """tile_offsets / total_tiles are accepted for the reference's call shape and unused:

@@ -40,9 +40,6 @@ int sy_router_route_rows(const void* h, const void* router, int N, int H, int E,
                          void* w, void* stream);
 // gemv.hip: the gate/up projection of a decode step that sorts its (at most 64) choices itself
 bool sy_gemv_sorts(int N, int k, int E, int H);
-int sy_grouped_gemv_sorting(const void* h, const int32_t* idx, const void* w, int N, int k, const void* gate_up, int E, int I,
-                            int H, int32_t* counts, int32_t* offsets, int32_t* token, void* wsorted, int32_t* pos_of,
-                            void* act, void* stream);
 // gemv.hip: the down projection and combine of a decode step (at most 8 tokens, 64 rows) in one launch
 bool sy_gemv_combines(int N, int k, int E, int H, int I);
 int sy_gemv_down_combine(const void* act, const void* down, const int32_t* offsets, const int32_t* token, const void* wsorted,

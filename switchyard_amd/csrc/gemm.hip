@@ -41,12 +41,17 @@ constexpr int LDS_LD = BK + 8;   // halves per LDS row (144 bytes)
 constexpr int GEMM_THREADS = 256;
 constexpr int XCDS = 8;
 
-// Inclusive prefix sum over the lanes of a wavefront.
-__device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
-  for (int o = 1; o < WAVE; o <<= 1) {
-    const int up = __shfl_up(v, o, WAVE);
-    if (lane >= o) v += up;
-  }
+// Inclusive prefix sum over the lanes of a wavefront, on DPP: shifts inside each row of 16 lanes,
+// then lane 15 of a row broadcast into the next row and lane 31 into the upper half. Six adds and
+// no trip through the LDS crossbar (a scan of shuffles is six dependent ds_bpermute, about 700
+// cycles, and the tile list of the stream kernel scans once per tile height).
+__device__ __forceinline__ int wave_inclusive_scan(int v, int /*lane*/) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);   // row_shr:1
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false);   // row_shr:2
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false);   // row_shr:4
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false);   // row_shr:8
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);   // row_bcast:15 into rows 1 and 3
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);   // row_bcast:31 into rows 2 and 3
   return v;
 }
 
@@ -75,7 +80,7 @@ __device__ __forceinline__ bool find_tile(const int* __restrict__ offsets, int E
       const int n = x < E ? offsets[x + 1] - offsets[x] : 0;
       row_tiles += (n + BM - 1) / BM;
     }
-    row_tiles = __shfl(wave_inclusive_scan(row_tiles, lane), WAVE - 1, WAVE);
+    row_tiles = __builtin_amdgcn_readlane(wave_inclusive_scan(row_tiles, lane), WAVE - 1);
     const long total = (long)row_tiles * ncol_tiles;
     const long per_xcd = (total + XCDS - 1) / XCDS;
     const long slot = blockIdx.x / XCDS;
@@ -102,7 +107,7 @@ __device__ __forceinline__ bool find_tile(const int* __restrict__ offsets, int E
           s_tile[2] = min(begin + height, last);
           s_tile[3] = col;
         }
-        run += __shfl(inc, WAVE - 1, WAVE);
+        run += __builtin_amdgcn_readlane(inc, WAVE - 1);
       }
     }
   }
@@ -475,7 +480,7 @@ gemm_stream_kernel(const half_t* __restrict__ A, const int* __restrict__ a_rows,
       const int mine = cls[s] == c ? tb.tiles[s] * ncol_tiles : 0;
       const int inc = wave_inclusive_scan(mine, lane);
       if (cls[s] == c) tb.lo[s] = run + inc - mine;
-      run += __shfl(inc, WAVE - 1, WAVE);
+      run += __builtin_amdgcn_readlane(inc, WAVE - 1);
     }
   }
   const int total = __builtin_amdgcn_readfirstlane(run);

@@ -595,9 +595,9 @@ gemv_down_combine_kernel(const half_t* __restrict__ act, const half_t* __restric
 // at most 64 choices happens inside the launch, whose first workgroup also writes the sort's
 // five results for the launches behind it. Same `act` as sy_sort_by_expert followed by
 // sy_grouped_gemv, bit for bit.
-int sy_grouped_gemv_sorting(const void* h, const int32_t* idx, const void* w, int N, int k, const void* gate_up, int E, int I,
-                            int H, int32_t* counts, int32_t* offsets, int32_t* token, void* wsorted, int32_t* pos_of,
-                            void* act, void* stream) {
+extern "C" SY_API int sy_grouped_gemv_sorting(const void* h, const int32_t* idx, const void* w, int N, int k, const void* gate_up,
+                                              int E, int I, int H, int32_t* counts, int32_t* offsets, int32_t* token,
+                                              void* wsorted, int32_t* pos_of, void* act, void* stream) {
   SY_REQUIRE(sy_gemv_sorts(N, k, E, H), "grouped_gemv_sorting: N = %d, k = %d, E = %d, H = %d", N, k, E, H);
   SY_REQUIRE((long)2 * I * H * 2 < (1l << 31) && I >= 1, "grouped_gemv_sorting: an expert's matrix must stay under 2 GiB");
   SY_REQUIRE(h && idx && w && gate_up && counts && offsets && token && wsorted && pos_of && act, "grouped_gemv_sorting: null pointer");
