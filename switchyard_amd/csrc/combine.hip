@@ -41,7 +41,7 @@ combine_kernel(const half_t* __restrict__ y, const int* __restrict__ pos_of, con
   for (int c = tid * 8; c < H; c += COMBINE_THREADS * 8) {
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     for (int j = 0; j < k; ++j) {
-      const half8_t v = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(y + (size_t)rows[j] * H + c));   // read once
+      const half8_t v = *reinterpret_cast<const half8_t*>(y + (size_t)rows[j] * H + c);
       const float wt = WEIGHTED ? weights[j] : 1.f;
 #pragma unroll
       for (int q = 0; q < 8; ++q) acc[q] += WEIGHTED ? (float)(half_t)((float)v[q] * wt) : (float)v[q];
