@@ -161,6 +161,29 @@ SY_API int sy_moe_experts(const void* h, const void* router, void* logits, int N
                           int32_t* pos_of, void* act, void* y, void* out, void* sort_workspace,
                           size_t sort_workspace_bytes, void* stream);
 
+/* Replaces moe_layer() (switchyard/kernels.py:91-93) in ONE call that takes one description of
+ * the layer and one scratch buffer: sy_moe_experts with the router given, the intermediate
+ * results (ids, weights, the sort's outputs, act, y, the sort's workspace, the logits) laid out by
+ * the library in `scratch`. A binding fills a SyMoeLayer once per (shape, weights) and then
+ * passes only h, out and the stream per call, which is what a call that is waited for wants:
+ * the host's time in front of the first launch is GPU idle time (switchyard/kernels.py:91-93 is
+ * two Python-level calls and a library GEMM in the reference).
+ * h f16 [N,H]; router f16 [E,H]; gate_up f16 [E,2I,H]; down f16 [E,H,I]; mfma_tiles 0 runs the
+ * weight-stream kernels, nonzero the MFMA tiles; scratch holds sy_moe_layer_scratch_bytes(N, E,
+ * k, H, I) bytes, 256-byte aligned, and is free again when the call's launches have run;
+ * out f16 [N,H]. Limits: those of sy_moe_experts with a router (E <= 128, k <= 8, H % 8 == 0 and
+ * H <= 8192, N*H*2 < 2 GiB). N == 0 is a no-op. */
+typedef struct SyMoeLayer {
+  int32_t N, E, k, norm, H, I, mfma_tiles, reserved;
+  const void* router;
+  const void* gate_up;
+  const void* down;
+  void* scratch;
+  size_t scratch_bytes;
+} SyMoeLayer;
+SY_API size_t sy_moe_layer_scratch_bytes(int N, int E, int k, int H, int I);
+SY_API int sy_moe_layer(const SyMoeLayer* layer, const void* h, void* out, void* stream);
+
 /* Replaces experts() (switchyard/kernels.py:76-88: sort -> pick -> ffn -> combine, for routing
  * computed elsewhere) in ONE call. idx int32 [N,k] and w f16 [N,k] are inputs; counts ... pos_of
  * are the sort's outputs as sy_sort_by_expert leaves them, act / y / out as in sy_moe_experts.

@@ -13,6 +13,7 @@ import collections
 import ctypes
 import threading
 import os
+import weakref
 
 import torch
 
@@ -20,6 +21,15 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libswitchyard_moe.so")
 
 _c_int, _c_void_p, _c_size_t, _c_float = ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_float
+
+
+class SyMoeLayer(ctypes.Structure):
+    """struct SyMoeLayer of include/switchyard_moe.h: one layer's shape, weights and scratch."""
+    _fields_ = [("N", ctypes.c_int32), ("E", ctypes.c_int32), ("k", ctypes.c_int32), ("norm", ctypes.c_int32),
+                ("H", ctypes.c_int32), ("I", ctypes.c_int32), ("mfma_tiles", ctypes.c_int32), ("reserved", ctypes.c_int32),
+                ("router", _c_void_p), ("gate_up", _c_void_p), ("down", _c_void_p), ("scratch", _c_void_p),
+                ("scratch_bytes", _c_size_t)]
+
 
 # name -> (restype, argtypes); mirrors include/switchyard_moe.h and include/switchyard_decode.h
 SIGNATURES = {
@@ -42,6 +52,8 @@ SIGNATURES = {
     "sy_combine": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p]),
     "sy_moe_experts": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p,
                                 _c_int, _c_int, _c_int, _c_int] + [_c_void_p] * 11 + [_c_size_t, _c_void_p]),
+    "sy_moe_layer_scratch_bytes": (_c_size_t, [_c_int, _c_int, _c_int, _c_int, _c_int]),
+    "sy_moe_layer": (_c_int, [ctypes.POINTER(SyMoeLayer), _c_void_p, _c_void_p, _c_void_p]),
     "sy_router_logits": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p]),
     "sy_router_route_sort": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int] + [_c_void_p] * 9),
     "sy_experts_sorted": (_c_int, [_c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int]
@@ -123,6 +135,9 @@ class Ext:
         self._plans = collections.OrderedDict()   # (shape, stream) -> plan; evicted least recently used first
         self._captured = {}                       # plans that a stream capture has seen: never evicted
         self._plans_lock = threading.Lock()
+        self._layers = {}                         # (N, ids of the weights, k, norm, tiles, stream) -> a prepared SyMoeLayer
+        self._scratch = collections.OrderedDict() # (bytes, device, stream) -> [alive, pinned, tensor] of moe_layer
+        self._scratch_pinned = []                 # scratch that a stream capture has seen: kept for good
 
     def _call(self, fn, *args):
         rc = fn(*args)
@@ -327,6 +342,82 @@ class Ext:
             return (starts, at, need, None, None)
         scratch = torch.empty(at, dtype=torch.uint8, device=device)
         return (starts, at, need, scratch, self._addresses(scratch, starts))
+
+    LAYERS_MAX = 1024   # prepared layer descriptions kept (a few hundred bytes each)
+
+    def moe_layer(self, h, router, gate_up, down, k, norm, mfma_tiles=False):
+        """moe_layer() of the reference in one call of the library (sy_moe_layer): h [N, H],
+        router [E, H], gate_up [E, 2I, H], down [E, H, I], all f16 -> out [N, H]. The description of
+        the layer (shape, weights, scratch) is prepared once per (token count, weights, stream)
+        and kept, so a call is a lookup, the allocation of `out` and one call with four arguments:
+        the host's time in front of the first launch is what a call that is waited for pays on
+        top of its kernels. The scratch is the per-(shape, stream) allocation of moe_experts, with
+        the same rules: calls on one stream share it, and one that a stream capture has seen is
+        never freed."""
+        if not (h.is_cuda and h.is_contiguous() and h.dtype == torch.float16 and h.dim() == 2):
+            raise RuntimeError("moe_layer: h must be a contiguous f16 GPU tensor [N, H]")
+        N = h.shape[0]
+        stream = _stream()
+        key = (N, id(router), id(gate_up), id(down), k, norm, mfma_tiles, stream)
+        with self._plans_lock:
+            entry = self._layers.get(key)
+            if entry is not None:
+                desc, plan, refs, ptrs = entry
+                if not (plan[0] and refs[0]() is router and refs[1]() is gate_up and refs[2]() is down and
+                        ptrs == (router.data_ptr(), gate_up.data_ptr(), down.data_ptr()) and desc.H == h.shape[1]):
+                    entry = None      # the scratch was evicted, or other tensors live at these ids now
+                elif not plan[1] and torch.cuda.is_current_stream_capturing():
+                    self._pin(plan)
+            if entry is None:
+                desc, plan = self._prepare_layer(h, router, gate_up, down, int(k), int(bool(norm)), bool(mfma_tiles), stream)
+                if len(self._layers) >= self.LAYERS_MAX:
+                    self._layers.clear()
+                self._layers[key] = (desc, plan, (weakref.ref(router), weakref.ref(gate_up), weakref.ref(down)),
+                                     (router.data_ptr(), gate_up.data_ptr(), down.data_ptr()))
+            out = torch.empty_like(h)
+            rc = self.lib.sy_moe_layer(desc, h.data_ptr(), out.data_ptr(), stream)
+        if rc:
+            raise RuntimeError(self.lib.sy_last_error().decode())
+        return out
+
+    def _pin(self, plan):
+        """A stream capture has seen this scratch: it leaves the least-recently-used list for good."""
+        plan[1] = True
+        for key, other in list(self._scratch.items()):
+            if other is plan:
+                del self._scratch[key]
+                self._scratch_pinned.append(plan)
+
+    def _prepare_layer(self, h, router, gate_up, down, k, norm, mfma_tiles, stream):
+        for t, name in ((router, "router"), (gate_up, "gate_up"), (down, "down")):
+            _check(t, name, torch.float16)
+        N, H = h.shape
+        E = router.shape[0]
+        if down.dim() != 3 or router.dim() != 2:
+            raise RuntimeError("moe_layer: router must be [E, H] and down [E, H, I]")
+        I = down.shape[2]
+        if tuple(router.shape) != (E, H) or tuple(gate_up.shape) != (E, 2 * I, H) or tuple(down.shape) != (E, H, I):
+            raise RuntimeError("moe_layer: shapes of h / router / gate_up / down do not match")
+        need = self.lib.sy_moe_layer_scratch_bytes(N, E, k, H, I)
+        skey = (need, h.device.index, stream)
+        plan = self._scratch.get(skey)          # [alive, pinned, tensor]
+        capturing = torch.cuda.is_current_stream_capturing()
+        if plan is None:
+            plan = [True, capturing, torch.empty(max(need, 256), dtype=torch.uint8, device=h.device)]
+            if capturing:
+                self._scratch_pinned.append(plan)
+            else:
+                if len(self._scratch) >= self.PLANS_MAX:
+                    _, old = self._scratch.popitem(last=False)
+                    old[0] = False              # descriptions that point at it are rebuilt on their next use
+                self._scratch[skey] = plan
+        else:
+            self._scratch.move_to_end(skey)
+            if capturing and not plan[1]:
+                self._pin(plan)
+        desc = SyMoeLayer(N, E, k, norm, H, I, int(mfma_tiles), 0, router.data_ptr(), gate_up.data_ptr(), down.data_ptr(),
+                          plan[2].data_ptr(), plan[2].numel())
+        return desc, plan
 
     def experts_routed(self, h, idx, w, gate_up, down, mfma_tiles=False):
         """experts() of the reference in one call of the library: h [N, H], idx int32 [N, k],

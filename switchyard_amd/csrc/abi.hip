@@ -104,6 +104,59 @@ extern "C" SY_API int sy_moe_experts(const void* h, const void* router, void* lo
                            stream);
 }
 
+// moe_layer() of the reference in one call with one scratch buffer: the layout of the
+// intermediate results is the library's business here.
+namespace {
+struct LayerScratch {
+  size_t idx, w, counts, offsets, token, wsorted, pos_of, act, y, sort_ws, logits, end, sort_bytes;
+};
+LayerScratch layer_scratch(int N, int E, int k, int H, int I) {
+  LayerScratch s;
+  size_t at = 0;
+  auto take = [&](size_t bytes) {
+    const size_t here = at;
+    at += (bytes + 255) / 256 * 256;
+    return here;
+  };
+  const size_t M = (size_t)N * k;
+  s.idx = take(M * 4);
+  s.w = take(M * 2);
+  s.counts = take((size_t)E * 4);
+  s.offsets = take((size_t)(E + 1) * 4);
+  s.token = take(M * 4);
+  s.wsorted = take(M * 2);
+  s.pos_of = take(M * 4);
+  s.act = take(M * I * 2);
+  s.y = take(M * H * 2);
+  s.sort_bytes = sy_sort_workspace_bytes(N, k, E);
+  s.sort_ws = take(s.sort_bytes);
+  s.logits = take((size_t)N * E * 2);
+  s.end = at;
+  return s;
+}
+}  // namespace
+
+extern "C" SY_API size_t sy_moe_layer_scratch_bytes(int N, int E, int k, int H, int I) {
+  if (N <= 0 || E <= 0 || k <= 0 || H <= 0 || I <= 0) return 0;
+  return layer_scratch(N, E, k, H, I).end;
+}
+
+extern "C" SY_API int sy_moe_layer(const SyMoeLayer* L, const void* h, void* out, void* stream) {
+  SY_REQUIRE(L, "moe_layer: null layer");
+  SY_REQUIRE(L->N >= 0 && L->E >= 1 && L->k >= 1 && L->H >= 8 && L->I >= 8, "moe_layer: N = %d, E = %d, k = %d, H = %d, I = %d",
+             L->N, L->E, L->k, L->H, L->I);
+  if (L->N == 0) return SY_OK;
+  SY_REQUIRE(L->router && L->gate_up && L->down && h && out, "moe_layer: null pointer");
+  const LayerScratch s = layer_scratch(L->N, L->E, L->k, L->H, L->I);
+  SY_REQUIRE(L->scratch && L->scratch_bytes >= s.end && ((uintptr_t)L->scratch & 255) == 0,
+             "moe_layer: scratch of %zu bytes, 256-byte aligned, needed (%zu given)", s.end, L->scratch_bytes);
+  char* b = (char*)L->scratch;
+  return sy_moe_experts(h, L->router, b + s.logits, L->N, L->E, L->k, L->norm, L->gate_up, L->down, L->H, L->I, L->mfma_tiles, 0,
+                        (int32_t*)(b + s.idx), b + s.w, (int32_t*)(b + s.counts), (int32_t*)(b + s.offsets),
+                        (int32_t*)(b + s.token), b + s.wsorted, (int32_t*)(b + s.pos_of), b + s.act, b + s.y, out,
+                        s.sort_bytes ? b + s.sort_ws : nullptr, s.sort_bytes, stream);
+}
+
 // experts() of the reference in one call: sort, the two projections, combine, from the routing.
 extern "C" SY_API int sy_experts_routed(const void* h, int N, int E, int k, const void* gate_up, const void* down, int H, int I,
                                         int mfma_tiles, const int32_t* idx, const void* w, int32_t* counts, int32_t* offsets,

@@ -188,16 +188,24 @@ OWN_ROUTER_MAX_TOKENS = 64
 def moe_layer(h, router, gate_up, down, top_k, norm_topk_prob, mode="auto"):
     N, n_experts = h.shape[0], gate_up.shape[0]
     if N > 0 and n_experts <= 128 and top_k <= 8 and h.dtype == torch.float16:
-        # one call of the library for everything after the router GEMM: the host pays for a call
-        # what the GPU needs for a small kernel, and the first projection would wait for it
         if mode == "auto":
             mode = _auto(N, N * top_k, n_experts)
         if mode not in ("gemv", "gemm", "cublas"):
             raise ValueError(f"unknown mode {mode!r}")
+        H = h.shape[1]
+        if (router.dtype == torch.float16 and H % 8 == 0 and H <= 8192 and N * H * 2 < 2 ** 31 and h.is_contiguous()
+                and router.is_contiguous()
+                and (N <= OWN_ROUTER_MAX_TOKENS or _abi.Ext.router_route_ok(N, H, n_experts, top_k))):
+            # one call of the library for the whole layer, the router's logits included: the host
+            # pays for a call what the GPU needs for a small kernel, and a layer that is waited
+            # for pays the host's time in front of its first launch in full
+            return ext().moe_layer(h, router, gate_up, down, top_k, norm_topk_prob, mode != "gemv")
+        # other shapes (a width the one-launch router does not take at more than 64 tokens, another
+        # dtype of the router): the library GEMM makes the logits, as in the reference (kernels.py:30-32)
         if N <= OWN_ROUTER_MAX_TOKENS:
-            own = h.shape[1] % 8 == 0 and h.shape[1] <= 8192
+            own = H % 8 == 0 and H <= 8192
         else:   # the router GEMM, route and the sort's first pass in one launch
-            own = router.dtype == torch.float16 and _abi.Ext.router_route_ok(N, h.shape[1], n_experts, top_k)
+            own = router.dtype == torch.float16 and _abi.Ext.router_route_ok(N, H, n_experts, top_k)
         return ext().moe_experts(h.contiguous(), None if own else F.linear(h, router).contiguous(), gate_up, down, top_k,
                                  norm_topk_prob, mfma_tiles=mode != "gemv", one_launch_front=N <= FUSED_FRONT_MAX_TOKENS,
                                  router=router.contiguous() if own else None)

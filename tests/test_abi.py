@@ -34,7 +34,7 @@ def test_header_declares_the_expected_entry_points():
     assert sorted(declared_symbols(HEADER)) == sorted(["sy_version", "sy_last_error", "sy_route", "sy_sort_workspace_bytes",
                                                   "sy_sort_by_expert", "sy_sort_by_expert_static", "sy_route_sort", "sy_router_route", "sy_experts_sorted", "sy_experts_routed",
                                                   "sy_grouped_gemv", "sy_grouped_gemv_sorting", "sy_grouped_gemm",
-                                                  "sy_combine", "sy_moe_experts"])
+                                                  "sy_combine", "sy_moe_experts", "sy_moe_layer", "sy_moe_layer_scratch_bytes"])
 
 
 def test_library_exports_every_declared_symbol(lib):
@@ -49,7 +49,7 @@ def test_each_header_citation_names_a_reference_location():
     text = open(HEADER).read()
     for name in ("sy_route", "sy_sort_by_expert", "sy_route_sort", "sy_grouped_gemv", "sy_grouped_gemv_sorting", "sy_grouped_gemm",
                  "sy_combine",
-                 "sy_moe_experts"):
+                 "sy_moe_experts", "sy_moe_layer"):
         comment = text[:text.index(f"SY_API int {name}(")].rsplit("/*", 1)[1]
         assert re.search(r"(moe_kernels\.cu|kernels\.py):\d+", comment), name
     # the entry point that allocates nothing replaces no reference interface and says so

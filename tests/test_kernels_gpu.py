@@ -751,35 +751,72 @@ def test_moe_experts_entry_point_with_a_width_the_mfma_front_does_not_take(K):
         assert torch.equal(out, K.experts(h, ridx, rw, gu, dn, "gemm" if tiles else "gemv"))
 
 
-def test_a_captured_layer_keeps_its_scratch_while_other_shapes_come_and_go(K):
-    """moe_layer keeps the intermediate results of small calls per (shape, stream) and drops the
+@pytest.mark.parametrize("path", ["layer", "experts"])
+def test_a_captured_layer_keeps_its_scratch_while_other_shapes_come_and_go(K, path):
+    """The binding keeps the intermediate results of small calls per (shape, stream) and drops the
     least recently used of them. A HIP graph captured through the call has the allocation's
     address in its kernel arguments, so that allocation must outlive any number of other shapes:
-    capture a layer of 8 tokens, run more other shapes than the binding keeps, replay."""
+    capture a layer of 8 tokens, run more other shapes than the binding keeps, replay. Both
+    bindings that keep scratch: moe_layer (one call of the library, the router given) and
+    moe_experts (the logits given)."""
     E, k, H, I = 64, 8, 512, 128
     _, router, gu, dn = (t.to(DEV) for t in cases.layer(1, E=E, k=k, H=H, I=I, seed=8, wstd=0.05))
-    h = hidden(8, H)
     ext = K.ext()
-    want = K.moe_layer(h, router, gu, dn, k, False).clone()
+    if path == "layer":
+        call = lambda x: K.moe_layer(x, router, gu, dn, k, False)
+        pinned, kept_lru = (lambda: len(ext._scratch_pinned)), (lambda: len(ext._scratch))
+    else:
+        call = lambda x: ext.moe_experts(x, F.linear(x, router).contiguous(), gu, dn, k, False, one_launch_front=True)
+        pinned, kept_lru = (lambda: len(ext._captured)), (lambda: len(ext._plans))
+    h = hidden(8, H)
+    want = call(h).clone()
     static_h = h.clone()
     torch.cuda.synchronize()
+    before = pinned()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
-        captured = K.moe_layer(static_h, router, gu, dn, k, False)
+        captured = call(static_h)
     graph.replay()
     torch.cuda.synchronize()
     assert torch.equal(captured, want)
-    kept = len(ext._captured)
-    assert kept >= 1
+    kept = pinned()
+    assert kept >= max(before, 1)
     others = []
     for n in range(9, 9 + ext.PLANS_MAX + 4):     # more shapes than the binding keeps
-        others.append(K.moe_layer(hidden(n, H), router, gu, dn, k, False))
+        others.append(call(hidden(n, H)))
     big = [torch.empty(32 << 20, dtype=torch.uint8, device=DEV).fill_(0xff) for _ in range(8)]   # reuse freed memory, if any
     torch.cuda.synchronize()
-    assert len(ext._plans) <= ext.PLANS_MAX and len(ext._captured) == kept
+    assert kept_lru() <= ext.PLANS_MAX and pinned() == kept
     for seed in (1, 2):
         static_h.copy_(hidden(8, H, seed=seed))
         graph.replay()
         torch.cuda.synchronize()
-        assert torch.equal(captured, K.moe_layer(static_h, router, gu, dn, k, False))
+        assert torch.equal(captured, call(static_h))
     del big, others
+
+
+def test_the_layer_in_one_call_equals_the_separate_calls(K):
+    """sy_moe_layer (one description of the layer, one scratch buffer) against route, sort, the
+    two projections and combine called one by one, at a decode size, at a size of the MFMA
+    tiles and at a width the MFMA front does not take; and the raw entry point refuses a
+    scratch buffer that is too small."""
+    ext = K.ext()
+    for N, E, k, H, I, mode in ((8, 64, 8, 512, 128, "gemv"), (3, 16, 4, 128, 64, "gemv"), (40, 64, 8, 512, 128, "gemm"),
+                                (300, 64, 8, 512, 64, "gemm"), (100, 16, 4, 768, 64, "gemm")):
+        h, router, gu, dn = (t.to(DEV) for t in cases.layer(N, E=E, k=k, H=H, I=I, seed=11, wstd=0.05))
+        got = ext.moe_layer(h, router, gu, dn, k, True, mode != "gemv")
+        if N <= K.OWN_ROUTER_MAX_TOKENS or not ext.router_route_ok(N, H, E, k):
+            logits = ext.router_logits(h, router)
+        else:
+            _, _, logits = ext.router_route(h, router, k, True)
+        idx, w = ext.route(logits, k, True)
+        assert torch.equal(got, K.experts(h, idx, w, gu, dn, mode)), (N, E, H, mode)
+        oidx, _ = O.route_logits(logits.cpu(), k, True)
+        assert torch.equal(idx.cpu().long(), oidx)
+    from switchyard_amd._abi import SyMoeLayer
+    need = ext.lib.sy_moe_layer_scratch_bytes(N, E, k, H, I)
+    small = torch.empty(need - 256, dtype=torch.uint8, device=DEV)
+    out = torch.empty_like(h)
+    desc = SyMoeLayer(N, E, k, 1, H, I, 1, 0, router.data_ptr(), gu.data_ptr(), dn.data_ptr(), small.data_ptr(), small.numel())
+    assert ext.lib.sy_moe_layer(desc, h.data_ptr(), out.data_ptr(), torch.cuda.current_stream().cuda_stream) == 1
+    assert b"scratch" in ext.lib.sy_last_error()
