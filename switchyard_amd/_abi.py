@@ -351,9 +351,10 @@ class Ext:
         the layer (shape, weights, scratch) is prepared once per (token count, weights, stream)
         and kept, so a call is a lookup, the allocation of `out` and one call with four arguments:
         the host's time in front of the first launch is what a call that is waited for pays on
-        top of its kernels. The scratch is the per-(shape, stream) allocation of moe_experts, with
-        the same rules: calls on one stream share it, and one that a stream capture has seen is
-        never freed."""
+        top of its kernels. The scratch is kept per (size, stream) up to PLAN_BYTES_MAX, with the
+        rules of moe_experts: calls on one stream share it, the least recently used of PLANS_MAX
+        goes first, and one that a stream capture has seen is never freed. Above that size the
+        scratch is allocated per call."""
         if not (h.is_cuda and h.is_contiguous() and h.dtype == torch.float16 and h.dim() == 2):
             raise RuntimeError("moe_layer: h must be a contiguous f16 GPU tensor [N, H]")
         N = h.shape[0]
@@ -370,10 +371,11 @@ class Ext:
                     self._pin(plan)
             if entry is None:
                 desc, plan = self._prepare_layer(h, router, gate_up, down, int(k), int(bool(norm)), bool(mfma_tiles), stream)
-                if len(self._layers) >= self.LAYERS_MAX:
-                    self._layers.clear()
-                self._layers[key] = (desc, plan, (weakref.ref(router), weakref.ref(gate_up), weakref.ref(down)),
-                                     (router.data_ptr(), gate_up.data_ptr(), down.data_ptr()))
+                if plan[0]:      # kept scratch: keep the description with it
+                    if len(self._layers) >= self.LAYERS_MAX:
+                        self._layers.clear()
+                    self._layers[key] = (desc, plan, (weakref.ref(router), weakref.ref(gate_up), weakref.ref(down)),
+                                         (router.data_ptr(), gate_up.data_ptr(), down.data_ptr()))
             out = torch.empty_like(h)
             rc = self.lib.sy_moe_layer(desc, h.data_ptr(), out.data_ptr(), stream)
         if rc:
@@ -399,6 +401,13 @@ class Ext:
         if tuple(router.shape) != (E, H) or tuple(gate_up.shape) != (E, 2 * I, H) or tuple(down.shape) != (E, H, I):
             raise RuntimeError("moe_layer: shapes of h / router / gate_up / down do not match")
         need = self.lib.sy_moe_layer_scratch_bytes(N, E, k, H, I)
+        if need > self.PLAN_BYTES_MAX:
+            # a large call: its scratch is this call's own (the allocator hands it on in stream order,
+            # and a capture keeps it in the graph's pool); nothing is kept, nothing can be evicted
+            scratch = torch.empty(need, dtype=torch.uint8, device=h.device)
+            desc = SyMoeLayer(N, E, k, norm, H, I, int(mfma_tiles), 0, router.data_ptr(), gate_up.data_ptr(),
+                              down.data_ptr(), scratch.data_ptr(), need)
+            return desc, [False, False, scratch]
         skey = (need, h.device.index, stream)
         plan = self._scratch.get(skey)          # [alive, pinned, tensor]
         capturing = torch.cuda.is_current_stream_capturing()
