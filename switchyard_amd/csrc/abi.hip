@@ -170,7 +170,7 @@ extern "C" SY_API int sy_experts_routed(const void* h, int N, int E, int k, cons
     // at most 64 choices: the gate/up stream sorts them in its own prologue
     rc = sy_grouped_gemv_sorting(h, idx, w, N, k, gate_up, E, I, H, counts, offsets, token, wsorted, pos_of, act, stream);
     if (rc) return rc;
-    // up to 8 tokens the down projection adds a token's rows up itself: no combine launch, no y
+    // up to 4 tokens the down projection adds a token's rows up itself: no combine launch, no y
     if (sy_gemv_combines(N, k, E, H, I)) return sy_gemv_down_combine(act, down, offsets, token, wsorted, N, k, E, H, I, out, stream);
     rc = sy_grouped_gemv(act, nullptr, down, offsets, E, N * k, N, H, I, 0, nullptr, y, stream);
     if (rc) return rc;
