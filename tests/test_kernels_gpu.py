@@ -596,6 +596,9 @@ def test_router_route_limits(K):
                                        (3000, 64, 8, 128, 64),         # the sort with a workspace
                                        # router GEMM and route in one launch (H a multiple of 512, above 64 tokens):
                                        (100, 64, 8, 512, 128), (300, 128, 8, 512, 64),
+                                       # ... with the router staged through LDS (H >= 1024, E <= 64), one workgroup sorting
+                                       (65, 16, 4, 1024, 64), (100, 64, 8, 1024, 64), (250, 60, 8, 1024, 64),
+                                       (256, 64, 8, 2048, 64), (511, 64, 4, 1024, 64),
                                        # ... which is also the sort's first pass above 2048 choices
                                        (1100, 64, 8, 512, 64), (2100, 16, 4, 512, 64), (1027, 60, 8, 1024, 64),
                                        # ... with two and four groups of 16 tokens to a piece of the sort
