@@ -419,6 +419,8 @@ class Ext:
                 if len(self._scratch) >= self.PLANS_MAX:
                     _, old = self._scratch.popitem(last=False)
                     old[0] = False              # descriptions that point at it are rebuilt on their next use
+                    old[2] = None               # ... and must not keep its memory meanwhile (what is queued on
+                                                # the stream it was allocated on runs before the memory is reused)
                 self._scratch[skey] = plan
         else:
             self._scratch.move_to_end(skey)
