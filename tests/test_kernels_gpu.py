@@ -708,6 +708,35 @@ def test_experts_from_the_routing_in_one_call(K, N, E, k, H, I, tiles):
             assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("N,E,k,H,I,routing", [(2, 64, 8, 2048, 1024, "routed"), (3, 64, 8, 2048, 1024, "routed"),
+                                               (4, 64, 8, 2048, 1024, "routed"), (4, 16, 4, 256, 512, "routed"),
+                                               (3, 128, 8, 512, 1024, "routed"), (4, 8, 8, 1024, 512, "routed"),
+                                               (4, 64, 8, 2048, 1024, "one expert"), (4, 16, 8, 256, 512, "two experts"),
+                                               (1, 4, 4, 8, 512, "routed")])
+def test_down_projection_and_combine_in_one_launch(K, N, E, k, H, I, routing):
+    """Up to 4 tokens (32 sorted rows) on the weight-stream kernels sy_experts_routed ends in one
+    launch that projects down and adds each token's rows up: `out` has the bits of the down
+    projection without scales followed by the combine that applies the router weights, and of
+    the plain separate calls. With ids that repeat inside a token (experts() takes any idx) an
+    expert has up to 32 rows."""
+    h, router, gu, dn = (t.to(DEV) for t in cases.layer(N, E=E, k=k, H=H, I=I, seed=12, wstd=0.05))
+    ext = K.ext()
+    assert ext.lib.sy_version() >= 200
+    idx, w = ext.route(F.linear(h, router).contiguous(), k, True)
+    if routing == "one expert":
+        idx = torch.full_like(idx, 5)
+    elif routing == "two experts":
+        idx = (torch.arange(N * k, device=DEV, dtype=torch.int32).reshape(N, k) % 2) * 9 + 3
+    counts, offsets, token, wsorted, pos_of = ext.sort_by_expert(idx, w, E)
+    M = N * k
+    act = ext.grouped_gemv(h, token, gu, offsets, M, True, None, M)
+    want = ext.combine(ext.grouped_gemv(act, None, dn, offsets, M, False, wsorted, M), pos_of, idx, N)
+    for _ in range(2):
+        assert torch.equal(ext.experts_routed(h, idx, w, gu, dn, mfma_tiles=False), want)
+    oracle = O.experts_loop(h.cpu().float(), idx.cpu().long(), w.cpu().float(), gu.cpu().float(), dn.cpu().float())
+    assert (want.cpu().float() - oracle).abs().max().item() <= 2e-2
+
+
 @pytest.mark.parametrize("N,E,k,H", [(1, 64, 8, 2048), (8, 64, 8, 2048), (64, 64, 8, 2048), (5, 100, 5, 520), (64, 128, 8, 8192)])
 def test_router_route_at_decode_sizes(K, N, E, k, H):
     """Up to 64 tokens sy_router_route is a workgroup per token: the logits of router_logits and
