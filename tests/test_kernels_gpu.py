@@ -513,6 +513,46 @@ def test_router_route_sort_counters_come_round(K):
             assert torch.equal(a, b), i
 
 
+def test_captured_router_route_sort_beside_eager_launches(K):
+    """A captured launch keeps its counter for every replay, so the library hands captured
+    launches counters that no launch outside a capture is ever given: a graph replays on one
+    stream while more eager launches than the pool's eager half holds run on another, and every
+    replay sorts as the three separate launches do."""
+    g = torch.Generator().manual_seed(21)
+    ext = K.ext()
+    cases = []
+    for N in (12, 40):
+        h = torch.randn(N, 1024, generator=g).half().to(DEV)
+        router = (torch.randn(64, 1024, generator=g) * 1024 ** -0.5).half().to(DEV)
+        logits = ext.router_logits(h, router)
+        idx, w = ext.route(logits, 8, True)
+        cases.append((h, router, [logits, idx, w] + list(ext.sort_by_expert(idx, w, 64))))
+    torch.cuda.synchronize()
+    side, other = torch.cuda.Stream(), torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        captured = [ext.router_route_sort(cases[0][0], cases[0][1], 8, True) for _ in range(3)]   # three counters
+    eager = []
+    for rep in range(40):
+        with torch.cuda.stream(side):
+            graph.replay()
+        with torch.cuda.stream(other):
+            for _ in range(15):     # 600 in all: the eager half of the pool comes round
+                eager.append(ext.router_route_sort(cases[1][0], cases[1][1], 8, True))
+        if rep % 8 == 7:
+            torch.cuda.synchronize()
+            for got in captured:
+                for a, b in zip(got, cases[0][2]):
+                    assert torch.equal(a, b), rep
+    torch.cuda.synchronize()
+    for got in captured:
+        for a, b in zip(got, cases[0][2]):
+            assert torch.equal(a, b)
+    for i, got in enumerate(eager):
+        for a, b in zip(got, cases[1][2]):
+            assert torch.equal(a, b), i
+
+
 def test_router_route_sort_on_two_streams_at_once(K):
     """Launches on different streams take different counters, so they may run side by side."""
     g = torch.Generator().manual_seed(9)
